@@ -160,6 +160,7 @@ void rope_cache(Tensor qkv, Tensor pos, Tensor cos_sin, c10::optional<Tensor> sl
 }
 
 // ------------------------------------------------------------------ MoE
+bool act_f32(const Tensor& t);   // defined with the fp32-stream ops below
 void moe_route(Tensor logits, int64_t k, Tensor ids, Tensor w) {
   CHECK_BF16(logits);
   TORCH_CHECK(logits.dim() == 2 && logits.stride(1) == 1, "moe_route: logits must be [T, E]");
@@ -180,7 +181,7 @@ void moe_align(Tensor ids, Tensor w, int64_t T, int64_t k, int64_t e0, int64_t E
   CHECK_DEV(sorted_w); CHECK_DT(sorted_w, at::kFloat);
   CHECK_DEV(inv); CHECK_DT(inv, at::kInt);
   CHECK_DEV(tiles); CHECK_DT(tiles, at::kInt);
-  TORCH_CHECK(E >= 1 && E <= 64 && (bm == 64 || bm == 128) && e0 >= 0);
+  TORCH_CHECK(E >= 1 && E <= 256 && (bm == 64 || bm == 128) && e0 >= 0);
   TORCH_CHECK(ids.numel() >= M && w.numel() >= M && sorted_tok.numel() >= M &&
               sorted_w.numel() >= M && inv.numel() >= M && tiles.numel() >= 3 * mt_cap);
   // every expert's rows fit the table: sum_e ceil(cnt_e / bm) <= M / bm + E
@@ -194,8 +195,10 @@ void moe_align(Tensor ids, Tensor w, int64_t T, int64_t k, int64_t e0, int64_t E
 
 // mode 0: out [M, F] = act(A[sorted_tok] @ W_e[:F]^T) * (A[sorted_tok] @ W_e[F:]^T)
 // mode 1: out [M, N] = (A @ W_e^T) * sorted_w
+// act 2: clamped GLU (limit, alpha); in_weight: the routing weight scales the gate | up accumulators (the
+// expert's input) and the down GEMM is left unscaled
 void moe_gemm(Tensor A, Tensor W, Tensor sorted_tok, Tensor sorted_w, Tensor tiles, int64_t mt,
-              int64_t bm, Tensor out, int64_t mode, int64_t act) {
+              int64_t bm, Tensor out, int64_t mode, int64_t act, double limit, double alpha, bool in_weight) {
   CHECK_BF16(A); CHECK_BF16(W); CHECK_BF16(out);
   CHECK_CONTIG(W); CHECK_CONTIG(out);
   CHECK_DEV(sorted_tok); CHECK_DT(sorted_tok, at::kInt);
@@ -232,8 +235,82 @@ void moe_gemm(Tensor A, Tensor W, Tensor sorted_tok, Tensor sorted_w, Tensor til
   p.tiles = tiles.data_ptr<int32_t>();
   p.out = bfp(out);
   p.ldo = out.stride(0);
+  TORCH_CHECK(act >= 0 && act <= 2);
   p.act = (int)act;
+  p.limit = (float)limit;
+  p.alpha = (float)alpha;
+  p.in_weight = in_weight ? 1 : 0;
   nga::launch_moe_gemm(p, (int)bm, (int)mode, cur_stream(out));
+}
+
+void moe_route_scores(Tensor logits, int64_t k, int64_t score, bool renorm, Tensor ids, Tensor w) {
+  CHECK_DEV(logits); CHECK_DT(logits, at::kFloat);
+  TORCH_CHECK(logits.dim() == 2 && logits.stride(1) == 1, "moe_route_scores: logits must be [T, E]");
+  const int64_t T = logits.size(0), E = logits.size(1);
+  TORCH_CHECK(E >= 1 && E <= 256 && k >= 1 && k <= 8 && k <= E, "moe_route_scores: 1 <= k <= min(8, E), E <= 256");
+  TORCH_CHECK(score == 0 || score == 1);
+  CHECK_DEV(ids); CHECK_DT(ids, at::kInt); CHECK_DEV(w); CHECK_DT(w, at::kFloat);
+  TORCH_CHECK(ids.is_contiguous() && w.is_contiguous() && ids.numel() >= T * k && w.numel() >= T * k);
+  nga::launch_moe_route_scores(logits.data_ptr<float>(), logits.stride(0), (int)T, (int)E, (int)k, (int)score, renorm,
+                               ids.data_ptr<int32_t>(), w.data_ptr<float>(), cur_stream(logits));
+}
+
+// the grouped GEMMs of moe_gemm on fp32-accumulating VALU tiles (bf16 or fp32, any sizes; 64-row M tiles).
+// mode 0: out [M, F] = clamped_glu(s (A[sorted_tok] W_e[:F]^T), s (A[sorted_tok] W_e[F:]^T)), s = sorted_w or 1
+// mode 1: out [M, N] = (A W_e^T) * (sorted_w or 1)
+void moe_gemm_rows(Tensor A, Tensor W, Tensor sorted_tok, Tensor sorted_w, Tensor tiles, int64_t mt, Tensor out,
+                   int64_t mode, double limit, double alpha, bool use_weight) {
+  const bool f32 = act_f32(A);
+  CHECK_CONTIG(W); CHECK_CONTIG(out);
+  TORCH_CHECK(W.is_cuda() && out.is_cuda() && W.scalar_type() == A.scalar_type() && out.scalar_type() == A.scalar_type());
+  CHECK_DEV(sorted_tok); CHECK_DT(sorted_tok, at::kInt);
+  CHECK_DEV(sorted_w); CHECK_DT(sorted_w, at::kFloat);
+  CHECK_DEV(tiles); CHECK_DT(tiles, at::kInt);
+  TORCH_CHECK(mode == 0 || mode == 1);
+  TORCH_CHECK(W.dim() == 3 && A.dim() == 2 && out.dim() == 2 && A.stride(1) == 1 && A.size(1) == W.size(2));
+  TORCH_CHECK(tiles.numel() >= 3 * mt && sorted_tok.numel() >= out.size(0) && sorted_w.numel() >= out.size(0));
+  nga::MoeRowsParams p{};
+  p.A = A.data_ptr();
+  p.lda = A.stride(0);
+  p.W = W.data_ptr();
+  p.w_rows = W.size(1);
+  p.K = (int)W.size(2);
+  p.mt = (int)mt;
+  if (mode == 0) {
+    TORCH_CHECK(W.size(1) % 2 == 0 && out.size(1) == W.size(1) / 2, "moe_gemm_rows: out must be [M, F]");
+    p.F = (int)(W.size(1) / 2);
+  } else {
+    TORCH_CHECK(out.size(1) == W.size(1) && A.size(0) >= out.size(0), "moe_gemm_rows: out must be [M, N]");
+    p.N = (int)W.size(1);
+  }
+  p.sorted_tok = sorted_tok.data_ptr<int32_t>();
+  p.sorted_w = sorted_w.data_ptr<float>();
+  p.tiles = tiles.data_ptr<int32_t>();
+  p.out = out.data_ptr();
+  p.ldo = out.stride(0);
+  p.limit = (float)limit;
+  p.alpha = (float)alpha;
+  p.use_weight = use_weight ? 1 : 0;
+  nga::launch_moe_gemm_rows(p, (int)mode, f32, cur_stream(out));
+}
+
+void moe_combine_rows(Tensor y, Tensor inv, int64_t T, int64_t k, c10::optional<Tensor> add, Tensor out) {
+  const bool f32 = act_f32(y);
+  CHECK_CONTIG(y); CHECK_CONTIG(out);
+  CHECK_DEV(inv); CHECK_DT(inv, at::kInt);
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == y.scalar_type());
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && y.dim() == 2 && y.size(1) == out.size(1));
+  TORCH_CHECK(inv.numel() >= T * k && y.size(0) >= T * k);
+  const void* ap = nullptr;
+  int64_t as = 0;
+  if (add.has_value()) {
+    TORCH_CHECK(add->is_cuda() && add->scalar_type() == y.scalar_type() && add->dim() == 2 && add->size(0) == T &&
+                add->size(1) == out.size(1) && add->stride(1) == 1, "add must be [T, H] rows");
+    ap = add->data_ptr();
+    as = add->stride(0);
+  }
+  nga::launch_moe_combine_rows(y.data_ptr(), inv.data_ptr<int32_t>(), (int)T, (int)k, (int)out.size(1), ap, as,
+                               out.data_ptr(), f32, cur_stream(y));
 }
 
 void moe_combine(Tensor y, Tensor inv, int64_t T, int64_t k, Tensor out) {
@@ -1163,10 +1240,97 @@ void relu_sq(Tensor out, Tensor x) {
   nga::launch_relu_sq(out.data_ptr(), x.data_ptr(), x.numel(), f32, cur_stream(x));
 }
 
-void softcap(Tensor z, double cap) {
+void softcap(Tensor z, double cap, double scale) {
   CHECK_F32(z);
   TORCH_CHECK(cap > 0);
-  nga::launch_softcap(z.data_ptr<float>(), z.numel(), (float)cap, cur_stream(z));
+  nga::launch_softcap(z.data_ptr<float>(), z.numel(), (float)cap, (float)scale, cur_stream(z));
+}
+
+void check_row_pages(const Tensor& act, const Tensor& c, int64_t heads, int64_t d, const char* what);
+const float* opt_f32(const c10::optional<Tensor>& t, int64_t n, const char* what);
+
+void residual_add_rmsnorm(Tensor x, Tensor y, c10::optional<Tensor> w, double eps, c10::optional<Tensor> out) {
+  CHECK_F32(x);
+  const bool f32 = act_f32(y);
+  const int64_t H = x.size(1);
+  TORCH_CHECK(x.dim() == 2 && y.dim() == 2 && y.size(0) == x.size(0) && y.size(1) == H && y.stride(1) == 1);
+  TORCH_CHECK(w.has_value() == out.has_value(), "residual_add_rmsnorm: a norm weight and its output come together");
+  void* op = nullptr;
+  if (out.has_value()) {
+    CHECK_CONTIG(*out);
+    TORCH_CHECK(out->is_cuda() && out->scalar_type() == y.scalar_type() && out->sizes() == x.sizes());
+    op = out->data_ptr();
+  }
+  nga::launch_residual_add_rmsnorm(x.data_ptr<float>(), y.data_ptr(), y.stride(0), opt_f32(w, H, "norm weight"),
+                                   (float)eps, x.size(0), (int)H, op, f32, cur_stream(x));
+}
+
+void clamped_glu(Tensor out, Tensor x, int64_t F, double limit, double alpha, int64_t gate_col) {
+  const bool f32 = act_f32(x);
+  CHECK_CONTIG(out);
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == x.scalar_type());
+  TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1 && F >= 1 && x.size(1) >= 2 * F && gate_col < x.size(1));
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == x.size(0) && out.size(1) == F);
+  nga::launch_clamped_glu(out.data_ptr(), x.data_ptr(), x.stride(0), x.size(0), (int)F, (float)limit, (float)alpha,
+                          (int)gate_col, f32, cur_stream(x));
+}
+
+void latent_rope_cache(Tensor proj, Tensor pos, Tensor slots, c10::optional<Tensor> page, Tensor freq, double mag,
+                       bool interleaved, int64_t rot_dims, int64_t rot_dim, double eps, int64_t kv_off, int64_t r,
+                       c10::optional<Tensor> kv_w, int64_t q_off, int64_t heads, int64_t dim,
+                       c10::optional<Tensor> q_out, int64_t n_off, int64_t n_n, c10::optional<Tensor> n_w) {
+  const bool f32 = act_f32(proj);
+  CHECK_I32(pos); CHECK_I32(slots);
+  const int64_t T = proj.size(0), W = proj.size(1);
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && pos.numel() == T && slots.numel() == T);
+  TORCH_CHECK(freq.is_cuda() && freq.scalar_type() == at::kDouble && freq.is_contiguous(), "freq: float64 on the GPU");
+  TORCH_CHECK(rot_dims >= 2 && rot_dims % 2 == 0 && rot_dims <= rot_dim && rot_dims <= 512 &&
+              freq.numel() == rot_dims / 2, "rotary positions: an even number of elements <= min(rot_dim, 512)");
+  nga::LatentRopeParams p{};
+  p.proj = proj.data_ptr();
+  p.stride = proj.stride(0);
+  p.pos = pos.data_ptr<int32_t>();
+  p.slots = slots.data_ptr<int32_t>();
+  p.freq = freq.data_ptr<double>();
+  p.mag = (float)mag;
+  p.eps = (float)eps;
+  p.interleaved = interleaved ? 1 : 0;
+  p.rot_dims = (int)rot_dims;
+  p.rot_dim = (int)rot_dim;
+  p.kv_off = -1;
+  p.q_off = -1;
+  p.n_off = -1;
+  if (kv_off >= 0) {
+    TORCH_CHECK(page.has_value() && r >= 1 && kv_off + r + rot_dim <= W, "latent columns outside the rows");
+    check_row_pages(proj, *page, 1, r + rot_dim, "latent_rope_cache");
+    p.page = page->data_ptr();
+    p.kv_off = (int)kv_off;
+    p.r = (int)r;
+    p.kv_w = opt_f32(kv_w, r, "latent norm weight");
+    TORCH_CHECK(p.kv_w != nullptr, "latent norm weight missing");
+  }
+  if (q_off >= 0) {
+    TORCH_CHECK(q_out.has_value() && heads >= 1 && dim >= 0 && q_off + heads * (dim + rot_dim) <= W,
+                "query heads outside the rows");
+    TORCH_CHECK(q_out->is_cuda() && q_out->scalar_type() == proj.scalar_type() && q_out->dim() == 2 &&
+                q_out->size(0) == T && q_out->stride(1) == 1 && q_out->size(1) % heads == 0 &&
+                q_out->size(1) / heads >= rot_dim, "q_out: [T, heads * W] rows of the activation type, W >= rot_dim");
+    p.q_off = (int)q_off;
+    p.heads = (int)heads;
+    p.dim = (int)dim;
+    p.q_out = q_out->data_ptr();
+    p.q_out_stride = q_out->stride(0);
+    p.q_w = (int)(q_out->size(1) / heads);
+  }
+  if (n_off >= 0) {
+    TORCH_CHECK(n_n >= 1 && n_off + n_n <= W, "norm columns outside the rows");
+    TORCH_CHECK(kv_off < 0 || n_off + n_n <= kv_off || n_off >= kv_off + r + rot_dim, "norm columns overlap the latent");
+    p.n_off = (int)n_off;
+    p.n_n = (int)n_n;
+    p.n_w = opt_f32(n_w, n_n, "norm weight");
+    TORCH_CHECK(p.n_w != nullptr, "norm weight missing");
+  }
+  nga::launch_latent_rope_cache(p, T, f32, cur_stream(proj));
 }
 
 void group_rmsnorm(Tensor out, Tensor x, Tensor w, int64_t groups, double eps) {
@@ -1229,7 +1393,7 @@ struct SoftmaxArgs {
 
 SoftmaxArgs check_softmax_args(const Tensor& out, const Tensor& q, const c10::optional<Tensor>& gate, const Tensor& kc,
                                const Tensor& vc, int64_t H, int64_t G, int64_t dk, int64_t dv, int64_t window,
-                               int64_t maps) {
+                               int64_t maps, bool v_in_k = false) {
   CHECK_CONTIG(out);
   TORCH_CHECK(out.is_cuda() && out.scalar_type() == q.scalar_type());
   const int64_t T = q.size(0);
@@ -1239,8 +1403,13 @@ SoftmaxArgs check_softmax_args(const Tensor& out, const Tensor& q, const c10::op
   TORCH_CHECK(H > 0 && G > 0 && H % G == 0 && dk > 0 && dk <= 2048 && dv > 0 && dv <= 512 && window >= 0,
               "softmax_attention: dk <= 2048, dv <= 512");
   check_row_pages(q, kc, G * maps, dk, "softmax_attention (k)");
-  check_row_pages(q, vc, G, dv, "softmax_attention (v)");
-  TORCH_CHECK(kc.size(0) == vc.size(0));
+  if (v_in_k) {
+    TORCH_CHECK(maps == 1 && dv <= dk && vc.data_ptr() == kc.data_ptr(),
+                "values inside the key rows: one map, dv <= dk, and the key pages passed as the value pages");
+  } else {
+    check_row_pages(q, vc, G, dv, "softmax_attention (v)");
+    TORCH_CHECK(kc.size(0) == vc.size(0));
+  }
   SoftmaxArgs a;
   if (gate.has_value()) {
     TORCH_CHECK(gate->is_cuda() && gate->scalar_type() == q.scalar_type() && gate->dim() == 2 && gate->size(0) == T &&
@@ -1253,17 +1422,17 @@ SoftmaxArgs check_softmax_args(const Tensor& out, const Tensor& q, const c10::op
 
 void softmax_attention(Tensor out, Tensor q, c10::optional<Tensor> gate, Tensor kc, Tensor vc, Tensor block_tables,
                        Tensor tok_seq, Tensor pos, int64_t H, int64_t G, int64_t dk, int64_t dv, double scale,
-                       int64_t window, int64_t maps, double lam, double unit_eps, double out_scale) {
+                       int64_t window, int64_t maps, double lam, double unit_eps, double out_scale, bool v_in_k) {
   const bool f32 = act_f32(q);
   CHECK_I32(block_tables); CHECK_I32(tok_seq); CHECK_I32(pos);
-  const SoftmaxArgs a = check_softmax_args(out, q, gate, kc, vc, H, G, dk, dv, window, maps);
+  const SoftmaxArgs a = check_softmax_args(out, q, gate, kc, vc, H, G, dk, dv, window, maps, v_in_k);
   const int64_t T = q.size(0);
   TORCH_CHECK(tok_seq.numel() == T && pos.numel() == T && block_tables.dim() == 2);
   nga::launch_softmax_attention(out.data_ptr(), q.data_ptr(), q.stride(0), a.gp, a.gs, kc.data_ptr(), vc.data_ptr(),
                                 block_tables.data_ptr<int32_t>(), (int)block_tables.size(1),
                                 tok_seq.data_ptr<int32_t>(), pos.data_ptr<int32_t>(), T, (int)H, (int)G, (int)dk,
                                 (int)dv, (float)scale, (int)window, (int)maps, (float)lam, (float)unit_eps,
-                                (float)out_scale, f32, cur_stream(q));
+                                (float)out_scale, v_in_k, f32, cur_stream(q));
 }
 
 // prompt portions on the MFMA kernel (bf16): sequence b owns rows [cu_q[b], cu_q[b + 1]) of q / gate / out,
@@ -1271,9 +1440,9 @@ void softmax_attention(Tensor out, Tensor q, c10::optional<Tensor> gate, Tensor 
 void softmax_attention_prefill(Tensor out, Tensor q, c10::optional<Tensor> gate, Tensor kc, Tensor vc,
                                Tensor block_tables, Tensor cu_q, Tensor ctx_lens, int64_t max_q_len, int64_t H,
                                int64_t G, int64_t dk, int64_t dv, double scale, int64_t window, int64_t maps, double lam,
-                               double unit_eps, double out_scale) {
+                               double unit_eps, double out_scale, bool v_in_k) {
   CHECK_BF16(q); CHECK_BF16(out); CHECK_I32(block_tables); CHECK_I32(cu_q); CHECK_I32(ctx_lens);
-  const SoftmaxArgs a = check_softmax_args(out, q, gate, kc, vc, H, G, dk, dv, window, maps);
+  const SoftmaxArgs a = check_softmax_args(out, q, gate, kc, vc, H, G, dk, dv, window, maps, v_in_k);
   TORCH_CHECK(nga::softmax_attention_mfma_supported((int)dk, (int)dv, (int)(H / G), (int)maps),
               "softmax_attention_prefill: head sizes the MFMA kernel does not take");
   TORCH_CHECK(q.stride(0) % 8 == 0 && (uintptr_t)q.data_ptr() % 16 == 0, "q rows must be 16-B aligned");
@@ -1283,16 +1452,16 @@ void softmax_attention_prefill(Tensor out, Tensor q, c10::optional<Tensor> gate,
                                      block_tables.data_ptr<int32_t>(), (int)block_tables.size(1),
                                      cu_q.data_ptr<int32_t>(), ctx_lens.data_ptr<int32_t>(), (int)B, (int)max_q_len,
                                      (int)H, (int)G, (int)dk, (int)dv, (float)scale, (int)window, (int)maps, (float)lam,
-                                     (float)unit_eps, (float)out_scale, cur_stream(q));
+                                     (float)unit_eps, (float)out_scale, v_in_k, cur_stream(q));
 }
 
 // single-token rows on the MFMA kernel (bf16): ws is the fp32 partial workspace [T, H, maps, parts, dv + 4]
 void softmax_attention_decode(Tensor out, Tensor ws, int64_t parts, Tensor q, c10::optional<Tensor> gate, Tensor kc,
                               Tensor vc, Tensor block_tables, Tensor tok_seq, Tensor pos, int64_t H, int64_t G,
                               int64_t dk, int64_t dv, double scale, int64_t window, int64_t maps, double lam,
-                              double unit_eps, double out_scale) {
+                              double unit_eps, double out_scale, bool v_in_k) {
   CHECK_BF16(q); CHECK_BF16(out); CHECK_F32(ws); CHECK_I32(block_tables); CHECK_I32(tok_seq); CHECK_I32(pos);
-  const SoftmaxArgs a = check_softmax_args(out, q, gate, kc, vc, H, G, dk, dv, window, maps);
+  const SoftmaxArgs a = check_softmax_args(out, q, gate, kc, vc, H, G, dk, dv, window, maps, v_in_k);
   TORCH_CHECK(nga::softmax_attention_mfma_supported((int)dk, (int)dv, (int)(H / G), (int)maps),
               "softmax_attention_decode: head sizes the MFMA kernel does not take");
   TORCH_CHECK(q.stride(0) % 8 == 0 && (uintptr_t)q.data_ptr() % 16 == 0, "q rows must be 16-B aligned");
@@ -1304,7 +1473,7 @@ void softmax_attention_decode(Tensor out, Tensor ws, int64_t parts, Tensor q, c1
                                   (const uint16_t*)a.gp, a.gs, bfp(kc), bfp(vc), block_tables.data_ptr<int32_t>(),
                                   (int)block_tables.size(1), tok_seq.data_ptr<int32_t>(), pos.data_ptr<int32_t>(), T,
                                   (int)H, (int)G, (int)dk, (int)dv, (float)scale, (int)window, (int)maps, (float)lam,
-                                  (float)unit_eps, (float)out_scale, cur_stream(q));
+                                  (float)unit_eps, (float)out_scale, v_in_k, cur_stream(q));
 }
 
 void hgrn2_scan(Tensor out, Tensor proj, Tensor f_bias, Tensor lower, Tensor state, int64_t H, int64_t d, int64_t dv,
@@ -1389,6 +1558,9 @@ PYBIND11_MODULE(_C, m) {
   m.def("rmsnorm_residual_next", checked("rmsnorm_residual_next", &rmsnorm_residual_next));
   m.def("relu_sq", checked("relu_sq", &relu_sq));
   m.def("softcap", checked("softcap", &softcap));
+  m.def("residual_add_rmsnorm", checked("residual_add_rmsnorm", &residual_add_rmsnorm));
+  m.def("clamped_glu", checked("clamped_glu", &clamped_glu));
+  m.def("latent_rope_cache", checked("latent_rope_cache", &latent_rope_cache));
   m.def("group_rmsnorm", checked("group_rmsnorm", &group_rmsnorm));
   m.def("headnorm_cache", checked("headnorm_cache", &headnorm_cache));
   m.def("softmax_attention", checked("softmax_attention", &softmax_attention));
@@ -1426,6 +1598,9 @@ PYBIND11_MODULE(_C, m) {
   m.def("moe_align", checked("moe_align", &moe_align));
   m.def("moe_gemm", checked("moe_gemm", &moe_gemm));
   m.def("moe_combine", checked("moe_combine", &moe_combine));
+  m.def("moe_route_scores", checked("moe_route_scores", &moe_route_scores));
+  m.def("moe_gemm_rows", checked("moe_gemm_rows", &moe_gemm_rows));
+  m.def("moe_combine_rows", checked("moe_combine_rows", &moe_combine_rows));
   m.def("skinny_cfg", &skinny_cfg);
   m.def("skinny_cfg_count", [] { return (int64_t)nga::skinny_gemm_cfg_count(); });
   m.def("skinny_gemm", checked("skinny_gemm", &skinny_gemm));

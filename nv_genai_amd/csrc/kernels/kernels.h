@@ -166,8 +166,30 @@ struct MoeGemmParams {
   const int32_t* tiles;      // [mt, 3]: expert, first row, end row (expert -1: unused)
   uint16_t* out;
   int64_t ldo;
-  int act;                   // MODE 0: 0 silu, 1 gelu_tanh
+  int act;                   // MODE 0: 0 silu, 1 gelu_tanh, 2 clamped GLU (limit, alpha)
+  float limit, alpha;
+  int in_weight;             // the routing weight scales the expert's input (MODE 0) and not its output (MODE 1)
 };
+// grouped GEMMs on fp32-accumulating VALU tiles: any sizes, bf16 or fp32 operands
+struct MoeRowsParams {
+  const void* A;             // MODE 0: token rows [T, K] (gathered); MODE 1: [M, K] sorted rows
+  int64_t lda;
+  const void* W;             // [E, w_rows, K]
+  int64_t w_rows;
+  int K, F, N, mt;           // MODE 0: F features (up rows start at F); MODE 1: N outputs
+  const int32_t* sorted_tok;
+  const float* sorted_w;
+  const int32_t* tiles;
+  void* out;
+  int64_t ldo;
+  float limit, alpha;
+  int use_weight;            // scale by the routing weight (MODE 0: gate and up before the activation)
+};
+void launch_moe_route_scores(const float* logits, int64_t ld, int T, int E, int k, int score, bool renorm,
+                             int32_t* ids, float* w, hipStream_t stream);
+void launch_moe_gemm_rows(const MoeRowsParams& p, int mode, bool f32, hipStream_t stream);
+void launch_moe_combine_rows(const void* y, const int32_t* inv, int T, int k, int H, const void* add,
+                             int64_t add_stride, void* out, bool f32, hipStream_t stream);
 void launch_moe_route(const uint16_t* logits, int64_t ld, int T, int E, int k, int32_t* ids,
                       float* w, hipStream_t stream);
 void launch_moe_align(const int32_t* ids, const float* w, int M, int k, int e0, int E, int bm,
@@ -267,7 +289,32 @@ void launch_embed_rows(float* x, const int32_t* ids, const void* embed, float sc
 void launch_rmsnorm_residual_next(float* x, const void* y, int64_t y_stride, const float* w, int w_n, const float* nw,
                                   int nw_n, float eps, int64_t T, int H, void* out, bool f32, hipStream_t stream);
 void launch_relu_sq(void* out, const void* in, int64_t n, bool f32, hipStream_t stream);
-void launch_softcap(float* z, int64_t n, float cap, hipStream_t stream);
+void launch_softcap(float* z, int64_t n, float cap, float scale, hipStream_t stream);
+void launch_residual_add_rmsnorm(float* x, const void* y, int64_t y_stride, const float* w, float eps, int64_t T, int H,
+                                 void* out, bool f32, hipStream_t stream);
+void launch_clamped_glu(void* out, const void* in, int64_t in_stride, int64_t T, int F, float limit, float alpha,
+                        int gate_col, bool f32, hipStream_t stream);
+
+// latent_rope.hip: latent norm + rotary positions + page write of latent attention with a rotated key part
+struct LatentRopeParams {
+  void* proj;                // [T, stride] projection rows (activation type)
+  int64_t stride;
+  const int32_t* pos;        // [T]
+  const int32_t* slots;      // [T] page slot of the token (< 0: no write)
+  void* page;                // [blocks, 1, 64, r + rot_dim] (nullptr with kv_off < 0)
+  const double* freq;        // [rot_dims / 2]
+  float mag, eps;
+  int interleaved, rot_dims, rot_dim;
+  int kv_off, r;             // latent columns [kv_off, kv_off + r), rotated key part behind them
+  const float* kv_w;         // [r]
+  int q_off, heads, dim;     // query heads of [dim | rot_dim] columns from q_off (q_off < 0: none)
+  void* q_out;               // [T, heads * q_w]; a head's rotated part goes to its last rot_dim columns
+  int64_t q_out_stride;
+  int q_w;
+  int n_off, n_n;            // in-place RMS norm of columns [n_off, n_off + n_n) (n_off < 0: none)
+  const float* n_w;
+};
+void launch_latent_rope_cache(const LatentRopeParams& p, int64_t T, bool f32, hipStream_t stream);
 void launch_group_rmsnorm(void* out, const float* x, const float* w, int64_t T, int groups, int gs, float eps, bool f32,
                           hipStream_t stream);
 
@@ -278,8 +325,8 @@ void launch_headnorm_cache(void* proj, int64_t stride, const int32_t* slots, voi
 void launch_softmax_attention(void* out, const void* q, int64_t q_stride, const void* gate, int64_t g_stride,
                               const void* kc, const void* vc, const int32_t* block_tables, int max_blocks,
                               const int32_t* tok_seq, const int32_t* pos, int64_t T, int H, int G, int dk, int dv,
-                              float scale, int window, int maps, float lam, float unit_eps, float out_scale, bool f32,
-                              hipStream_t stream);
+                              float scale, int window, int maps, float lam, float unit_eps, float out_scale, bool v_in_k,
+                              bool f32, hipStream_t stream);
 
 bool softmax_attention_mfma_supported(int dk, int dv, int group, int maps);
 void launch_softmax_attention_mfma(uint16_t* out, const uint16_t* q, int64_t q_stride, const uint16_t* gate,
@@ -287,13 +334,14 @@ void launch_softmax_attention_mfma(uint16_t* out, const uint16_t* q, int64_t q_s
                                    const int32_t* block_tables, int max_blocks, const int32_t* cu_q,
                                    const int32_t* ctx_lens, int B, int max_q_len, int H, int G, int dk, int dv,
                                    float scale, int window, int maps, float lam, float unit_eps, float out_scale,
-                                   hipStream_t stream);
+                                   bool v_in_k, hipStream_t stream);
 int softmax_decode_parts(int rows, int G, int max_ctx, int window);
 void launch_softmax_decode_mfma(uint16_t* out, float* ws, int parts, const uint16_t* q, int64_t q_stride,
                                 const uint16_t* gate, int64_t g_stride, const uint16_t* kc, const uint16_t* vc,
                                 const int32_t* block_tables, int max_blocks, const int32_t* tok_seq,
                                 const int32_t* pos, int64_t T, int H, int G, int dk, int dv, float scale, int window,
-                                int maps, float lam, float unit_eps, float out_scale, hipStream_t stream);
+                                int maps, float lam, float unit_eps, float out_scale, bool v_in_k,
+                                hipStream_t stream);
 
 // recurrent.hip
 int hgrn2_max_dim(int dv);

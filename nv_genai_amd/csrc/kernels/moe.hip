@@ -11,6 +11,18 @@
 //                rows and scales by the routing weight
 //   moe_combine  sums each token's top-k rows (fp32) into [T, H]
 //
+// Routing and experts of other designs (same align / tile table, same order of steps):
+//   moe_route_scores  fp32 router logits -> top-k ids + weights, sigmoid or softmax scores, as
+//                they are or renormalised over the k
+//   moe_gemm act 2    clamped GLU epilogue g sigmoid(alpha g) (u + 1), g = min(gate, limit),
+//                u = clamp(up, +-limit), with the routing weight on the expert's input
+//                (the accumulators are scaled: W (s x) = s (W x)) and none on the down GEMM
+//   moe_gemm_rows     the grouped GEMMs on 64 x 64 fp32-accumulating VALU tiles: bf16 or fp32
+//                operands, any K / F / N (experts too small or too odd for the MFMA tiles,
+//                and the true-fp32 path)
+//   moe_combine_rows  moe_combine for any width and type, plus an optional added row (a shared
+//                expert's output)
+//
 // GEMM: see the block comment above moe_gemm_kernel. Weight rows are the MFMA A operand and
 // token rows the B operand, so each lane
 // ends with 4 consecutive output features of one token: 8-byte stores, and in MODE 0 the
@@ -26,7 +38,7 @@ namespace nga {
 
 namespace {
 constexpr int BK = 64;   // K per stage (one 128-B row of bf16)
-constexpr int MAX_E = 64;
+constexpr int MAX_E = 256;
 
 __device__ __forceinline__ int swz(int row, int ch) {  // 16-B chunk position in a 128-B LDS row
   return row * BK + ((ch ^ ((row >> 1) & 7)) << 3);
@@ -36,6 +48,12 @@ __device__ __forceinline__ float silu(float x) { return x / (1.f + __expf(-x)); 
 __device__ __forceinline__ float gelu_tanh(float x) {
   const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
   return x - x / (1.f + __expf(2.f * u));
+}
+// g sigmoid(alpha g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit)
+__device__ __forceinline__ float clamped_glu(float gate, float up, float limit, float alpha) {
+  const float g = fminf(gate, limit);
+  const float u = fminf(fmaxf(up, -limit), limit);
+  return g / (1.f + expf(-alpha * g)) * (u + 1.f);
 }
 }  // namespace
 
@@ -283,19 +301,21 @@ __global__ void __launch_bounds__(256) moe_gemm_kernel(MoeGemmParams P) {
     if (pos >= row1) continue;
     uint16_t* op = P.out + (int64_t)pos * P.ldo;
     if (MODE == 0) {
+      const float sw = P.in_weight ? P.sorted_w[pos] : 1.f;   // W (s x) = s (W x)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int f = nb * 128 + wn * 64 + g * 16 + 4 * h;
         u16x4 v;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const float gt = acc[2 * g][mt][r], up = acc[2 * g + 1][mt][r];
-          v[r] = f2bf((P.act == 0 ? silu(gt) : gelu_tanh(gt)) * up);
+          const float gt = acc[2 * g][mt][r] * sw, up = acc[2 * g + 1][mt][r] * sw;
+          v[r] = f2bf(P.act == 2 ? clamped_glu(gt, up, P.limit, P.alpha)
+                                 : (P.act == 0 ? silu(gt) : gelu_tanh(gt)) * up);
         }
         *reinterpret_cast<u16x4*>(op + f) = v;
       }
     } else {
-      const float sc = P.sorted_w[pos];
+      const float sc = P.in_weight ? 1.f : P.sorted_w[pos];
 #pragma unroll
       for (int nt = 0; nt < NTW; ++nt) {
         const int n = nb * BN + wn * 128 + nt * 16 + 4 * h;
@@ -330,6 +350,158 @@ __global__ void moe_combine_kernel(const uint16_t* __restrict__ y, const int32_t
 #pragma unroll
     for (int q = 0; q < 8; ++q) o[q] = f2bf(a[q]);
     store8(out + t * H + c, o);
+  }
+}
+
+// ------------------------------------------------------------------ routing from fp32 logits
+// One thread per token. score 0: sigmoid(logit); 1: softmax probability over all experts. The
+// k largest scores in descending order (ties: the lower expert index), chosen by the logits -
+// the scores are monotonic in them, so rounding of the score cannot reorder a pair. Weights as
+// they are or divided by their sum over the k.
+__global__ void moe_route_scores_kernel(const float* __restrict__ logits, int64_t ld, int T, int E, int k, int score,
+                                        int renorm, int32_t* __restrict__ ids, float* __restrict__ w) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const float* lp = logits + (int64_t)t * ld;
+  float top[8];
+  int sel[8];
+  for (int j = 0; j < k; ++j) {
+    float best = -INFINITY;
+    int bi = -1;
+    for (int e = 0; e < E; ++e) {
+      bool taken = false;
+      for (int i = 0; i < j; ++i) taken |= sel[i] == e;
+      const float v = lp[e];
+      if (!taken && (bi < 0 || v > best)) {
+        best = v;
+        bi = e;
+      }
+    }
+    top[j] = best;
+    sel[j] = bi;
+  }
+  const float mx = top[0];
+  float den = 1.f;
+  if (score == 1) {
+    den = 0.f;
+    for (int e = 0; e < E; ++e) den += expf(lp[e] - mx);
+  }
+  float sum = 0.f;
+  for (int j = 0; j < k; ++j) {
+    top[j] = score == 0 ? 1.f / (1.f + expf(-top[j])) : expf(top[j] - mx) / den;
+    sum += top[j];
+  }
+  for (int j = 0; j < k; ++j) {
+    ids[(int64_t)t * k + j] = sel[j];
+    w[(int64_t)t * k + j] = renorm ? top[j] / sum : top[j];
+  }
+}
+
+// ------------------------------------------------------------------ grouped GEMM on VALU tiles
+// Workgroup (256 threads) = one M tile of the table (<= 64 sorted rows of one expert) x 64
+// output columns; K in steps of 16 through LDS; a thread owns 4 rows x 4 columns (fp32). MODE 0:
+// gathered token rows x the expert's gate and up rows of the same 64 features (two accumulator
+// sets), epilogue = routing weight on the input (optional) and the clamped GLU; MODE 1: sorted
+// activation rows x the expert's down rows, optionally times the routing weight. No alignment
+// or divisibility is assumed.
+namespace {
+template <typename T> __device__ __forceinline__ float ldv(const T* p);
+template <> __device__ __forceinline__ float ldv<uint16_t>(const uint16_t* p) { return bf2f(*p); }
+template <> __device__ __forceinline__ float ldv<float>(const float* p) { return *p; }
+template <typename T> __device__ __forceinline__ void stv(T* p, float v);
+template <> __device__ __forceinline__ void stv<uint16_t>(uint16_t* p, float v) { *p = f2bf(v); }
+template <> __device__ __forceinline__ void stv<float>(float* p, float v) { *p = v; }
+constexpr int RT = 64, RK = 16;
+}  // namespace
+
+template <typename T, int MODE>
+__global__ void __launch_bounds__(256) moe_gemm_rows_kernel(MoeRowsParams P) {
+  __shared__ float xs[RK][RT + 1];          // [k][row]
+  __shared__ float wsA[RK][RT + 1];         // [k][col]: gate (MODE 0) / down rows
+  __shared__ float wsB[MODE == 0 ? RK : 1][RT + 1];   // up rows
+  const int mti = blockIdx.y, nb = blockIdx.x;
+  const int e = P.tiles[3 * mti];
+  if (e < 0) return;
+  const int row0 = P.tiles[3 * mti + 1], row1 = P.tiles[3 * mti + 2];
+  const int tid = threadIdx.x;
+  const int tr = tid >> 4, tc = tid & 15;    // rows 4 tr .. + 3, columns 4 tc .. + 3
+  const int N = MODE == 0 ? P.F : P.N;
+  const T* A = (const T*)P.A;
+  const T* We = (const T*)P.W + (int64_t)e * P.w_rows * P.K;
+  // staging: thread loads element (r = tid / 16 + 16 i, k = tid % 16) of the x and w tiles
+  const int lk = tid & 15, lr = tid >> 4;
+  float accA[4][4], accB[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) accA[i][j] = accB[i][j] = 0.f;
+  int64_t arow[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int pos = row0 + lr + 16 * i;
+    arow[i] = pos < row1 ? (MODE == 0 ? (int64_t)P.sorted_tok[pos] : (int64_t)pos) : -1;
+  }
+  for (int k0 = 0; k0 < P.K; k0 += RK) {
+    const int kk = k0 + lk;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = lr + 16 * i;
+      xs[lk][r] = (arow[i] >= 0 && kk < P.K) ? ldv(A + arow[i] * P.lda + kk) : 0.f;
+      const int n = nb * RT + r;
+      const bool ok = n < N && kk < P.K;
+      wsA[lk][r] = ok ? ldv(We + (int64_t)n * P.K + kk) : 0.f;
+      if (MODE == 0) wsB[lk][r] = ok ? ldv(We + (int64_t)(P.F + n) * P.K + kk) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < RK; ++k) {
+      float xv[4], wa[4], wb[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) xv[i] = xs[k][4 * tr + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        wa[j] = wsA[k][4 * tc + j];
+        if (MODE == 0) wb[j] = wsB[k][4 * tc + j];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          accA[i][j] += xv[i] * wa[j];
+          if (MODE == 0) accB[i][j] += xv[i] * wb[j];
+        }
+    }
+    __syncthreads();
+  }
+  T* out = (T*)P.out;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int pos = row0 + 4 * tr + i;
+    if (pos >= row1) continue;
+    const float sw = P.use_weight ? P.sorted_w[pos] : 1.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = nb * RT + 4 * tc + j;
+      if (n >= N) continue;
+      const float v = MODE == 0 ? clamped_glu(accA[i][j] * sw, accB[i][j] * sw, P.limit, P.alpha) : accA[i][j] * sw;
+      stv(out + (int64_t)pos * P.ldo + n, v);
+    }
+  }
+}
+
+// out[t, :] = sum_j y[inv[t*k + j], :] (+ add[t, :]) in fp32, any width
+template <typename T>
+__global__ void __launch_bounds__(256) moe_combine_rows_kernel(const T* __restrict__ y, const int32_t* __restrict__ inv,
+                                                               int k, int H, const T* __restrict__ add,
+                                                               int64_t add_stride, T* __restrict__ out) {
+  const int64_t t = blockIdx.x;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    float a = add ? ldv(add + t * add_stride + c) : 0.f;
+    for (int j = 0; j < k; ++j) {
+      const int p = inv[t * k + j];
+      if (p >= 0) a += ldv(y + (int64_t)p * H + c);
+    }
+    stv(out + t * H + c, a);
   }
 }
 
@@ -372,6 +544,36 @@ void launch_moe_gemm(const MoeGemmParams& p, int bm, int mode, hipStream_t strea
     if (bm == 64) moe_gemm_kernel<64, 1><<<grid, 256, 0, stream>>>(p);
     else moe_gemm_kernel<128, 1><<<grid, 256, 0, stream>>>(p);
   }
+}
+
+void launch_moe_route_scores(const float* logits, int64_t ld, int T, int E, int k, int score, bool renorm,
+                             int32_t* ids, float* w, hipStream_t stream) {
+  if (T == 0) return;
+  moe_route_scores_kernel<<<(T + 127) / 128, 128, 0, stream>>>(logits, ld, T, E, k, score, renorm ? 1 : 0, ids, w);
+}
+
+void launch_moe_gemm_rows(const MoeRowsParams& p, int mode, bool f32, hipStream_t stream) {
+  const int N = mode == 0 ? p.F : p.N;
+  if (p.mt == 0 || N == 0) return;
+  dim3 grid((N + RT - 1) / RT, p.mt);
+  if (f32) {
+    if (mode == 0) moe_gemm_rows_kernel<float, 0><<<grid, 256, 0, stream>>>(p);
+    else moe_gemm_rows_kernel<float, 1><<<grid, 256, 0, stream>>>(p);
+  } else {
+    if (mode == 0) moe_gemm_rows_kernel<uint16_t, 0><<<grid, 256, 0, stream>>>(p);
+    else moe_gemm_rows_kernel<uint16_t, 1><<<grid, 256, 0, stream>>>(p);
+  }
+}
+
+void launch_moe_combine_rows(const void* y, const int32_t* inv, int T, int k, int H, const void* add,
+                             int64_t add_stride, void* out, bool f32, hipStream_t stream) {
+  if (T == 0) return;
+  if (f32)
+    moe_combine_rows_kernel<float><<<T, 256, 0, stream>>>((const float*)y, inv, k, H, (const float*)add, add_stride,
+                                                         (float*)out);
+  else
+    moe_combine_rows_kernel<uint16_t><<<T, 256, 0, stream>>>((const uint16_t*)y, inv, k, H, (const uint16_t*)add,
+                                                            add_stride, (uint16_t*)out);
 }
 
 void launch_moe_combine(const uint16_t* y, const int32_t* inv, int T, int k, int H, uint16_t* out,

@@ -11,7 +11,11 @@
 //                     post-norm of one sub-layer and the pre-norm of the next in one pass
 //                     (weights of H elements or of one: a single gain)
 //   relu_sq           relu(x)^2
-//   softcap           z = cap * tanh(z / cap) on fp32 logits
+//   softcap           z = cap * tanh(z * scale / cap) on fp32 logits
+//   residual_add_rmsnorm   x[t] += y[t], out[t] = rmsnorm(x[t]) * w: the residual sum of one
+//                     pre-norm sub-layer and the norm in front of the next in one pass
+//   clamped_glu       [gate F | up F | ...] -> g sigmoid(alpha g) (u + 1), g = min(gate, limit),
+//                     u = clamp(up, +-limit), optionally times sigmoid of one gate column of the row
 //   group_rmsnorm     RMS norm of each of G equal column groups of fp32 rows (heads)
 //
 // The residual, the norms and the shift interpolation are fp32 whatever the activation type T
@@ -184,6 +188,45 @@ __global__ void __launch_bounds__(256) relu_sq_bf16x8_kernel(uint16_t* __restric
   }
 }
 
+// Two passes over the row: residual sum with the statistic of the new x, then the norm's output
+// (each thread re-reads only the columns it wrote itself). out == nullptr: the sum only.
+template <typename T>
+__global__ void __launch_bounds__(256) residual_add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ y,
+                                                                   int64_t y_stride, const float* __restrict__ w,
+                                                                   float eps, int H, T* __restrict__ out) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const T* yr = y + row * y_stride;
+  float* xr = x + row * H;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    const float v = xr[c] + ldf(yr + c);
+    xr[c] = v;
+    ss += v * v;
+  }
+  if (!out) return;
+  ss = block_sum(ss, red);
+  const float r = 1.0f / sqrtf(ss / (float)H + eps);
+  for (int c = threadIdx.x; c < H; c += blockDim.x) stf(out + row * H + c, xr[c] * r * w[c]);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) clamped_glu_kernel(T* __restrict__ out, const T* __restrict__ in,
+                                                          int64_t in_stride, int64_t T_rows, int F, float limit,
+                                                          float alpha, int gate_col) {
+  const int64_t total = T_rows * F;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = i / F;
+    const int c = (int)(i - t * F);
+    const T* r = in + t * in_stride;
+    const float g = fminf(ldf(r + c), limit);
+    const float u = fminf(fmaxf(ldf(r + F + c), -limit), limit);
+    float v = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+    if (gate_col >= 0) v *= 1.0f / (1.0f + expf(-ldf(r + gate_col)));
+    stf(out + i, v);
+  }
+}
+
 __global__ void __launch_bounds__(256) softcap_kernel(float* __restrict__ z, int64_t n, float cap, float inv) {
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
     z[i] = cap * tanhf(z[i] * inv);
@@ -300,11 +343,35 @@ void launch_relu_sq(void* out, const void* in, int64_t n, bool f32, hipStream_t 
     relu_sq_kernel<uint16_t><<<dim3((unsigned)g), 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)in, n);
 }
 
-void launch_softcap(float* z, int64_t n, float cap, hipStream_t stream) {
+void launch_softcap(float* z, int64_t n, float cap, float scale, hipStream_t stream) {
   if (n == 0) return;
   int64_t g = (n + 255) / 256;
   if (g > 16384) g = 16384;
-  softcap_kernel<<<dim3((unsigned)g), 256, 0, stream>>>(z, n, cap, 1.0f / cap);
+  softcap_kernel<<<dim3((unsigned)g), 256, 0, stream>>>(z, n, cap, scale / cap);
+}
+
+void launch_residual_add_rmsnorm(float* x, const void* y, int64_t y_stride, const float* w, float eps, int64_t T, int H,
+                                 void* out, bool f32, hipStream_t stream) {
+  if (T == 0) return;
+  if (f32)
+    residual_add_rmsnorm_kernel<float><<<dim3((unsigned)T), 256, 0, stream>>>(x, (const float*)y, y_stride, w, eps, H,
+                                                                             (float*)out);
+  else
+    residual_add_rmsnorm_kernel<uint16_t><<<dim3((unsigned)T), 256, 0, stream>>>(x, (const uint16_t*)y, y_stride, w, eps,
+                                                                                H, (uint16_t*)out);
+}
+
+void launch_clamped_glu(void* out, const void* in, int64_t in_stride, int64_t T, int F, float limit, float alpha,
+                        int gate_col, bool f32, hipStream_t stream) {
+  if (T == 0 || F == 0) return;
+  int64_t g = (T * F + 255) / 256;
+  if (g > 8192) g = 8192;
+  if (f32)
+    clamped_glu_kernel<float><<<dim3((unsigned)g), 256, 0, stream>>>((float*)out, (const float*)in, in_stride, T, F,
+                                                                    limit, alpha, gate_col);
+  else
+    clamped_glu_kernel<uint16_t><<<dim3((unsigned)g), 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)in, in_stride,
+                                                                       T, F, limit, alpha, gate_col);
 }
 
 void launch_group_rmsnorm(void* out, const float* x, const float* w, int64_t T, int groups, int gs, float eps, bool f32,

@@ -19,7 +19,9 @@
 // its keys are k head (h / (H / G)) * maps + m. Two maps combine as a_0 - lam * a_1
 // (differential attention). Optional: unit RMS of the head output (eps inside the root) times
 // out_scale, and a per-head sigmoid gate. Visible keys of the query at position i: j <= i, and
-// i - j < window when window > 0.
+// i - j < window when window > 0. v_row: elements between two value rows of a page; v_row = dk with
+// vc = kc reads the values out of the first dv elements of the key rows (one map: a latent that is
+// key and value, followed by key-only columns).
 #include <cstdlib>
 
 #include "common.h"
@@ -124,7 +126,7 @@ __global__ void __launch_bounds__(64) softmax_attention_kernel(
     T* __restrict__ out, const T* __restrict__ q, int64_t q_stride, const T* __restrict__ gate, int64_t g_stride,
     const T* __restrict__ kc, const T* __restrict__ vc, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int H, int G, int dk, int dv, float scale,
-    int window, int maps, float lam, float unit_eps, float out_scale) {
+    int window, int maps, float lam, float unit_eps, float out_scale, int v_row) {
   extern __shared__ float smem[];
   float* qs = smem;                 // [maps * dk]
   float* ws = smem + maps * dk;     // [64]
@@ -167,13 +169,13 @@ __global__ void __launch_bounds__(64) softmax_attention_kernel(
       __syncthreads();
       const unsigned long long any = __ballot(vis);
       const int j0 = __builtin_ctzll(any), j1 = 63 - __builtin_clzll(any);
-      const T* vp = vc + ((page * G + g) * BS) * (int64_t)dv;
+      const T* vp = vc + ((page * G + g) * BS) * (int64_t)v_row;
 #pragma unroll
       for (int u = 0; u < MAXV; ++u) {
         const int d = lane + u * 64;
         if (d < dv) {
           float a = acc[u] * corr;
-          for (int jj = j0; jj <= j1; ++jj) a += ws[jj] * ldf(vp + (int64_t)jj * dv + d);
+          for (int jj = j0; jj <= j1; ++jj) a += ws[jj] * ldf(vp + (int64_t)jj * v_row + d);
           acc[u] = a;
         }
       }
@@ -226,6 +228,7 @@ struct SmMfmaParams {
   int64_t q_stride, g_stride;
   int max_blocks, H, G, window;
   float scale_log2, lam, unit_eps, out_scale;
+  int v_row;                 // elements between value rows of a page (DV, or DK when the values lie in the key rows)
 };
 
 // WPE: waves per SIMD the register allocation aims at. Large tiles (maps x DK + DV >= 192) are
@@ -240,7 +243,10 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
   constexpr int DT = DV / 16;
   constexpr int PER_K = DK / 32;           // 16-B chunks per thread per K page
   constexpr int VBLK = (2 * DV + 255) / 256;   // (4 keys x 8 columns) blocks per thread per V page
-  constexpr int SWS = NCH_K >= 16 ? 0 : NCH_K == 8 ? 1 : 2;
+  // the XOR must stay inside an aligned group of chunks that the row holds whole: the largest
+  // power of two dividing the chunk count (96-, 192-, 320-wide keys: 4, 8, 8 chunks)
+  constexpr int P2 = NCH_K & -NCH_K;
+  constexpr int SWS = P2 >= 16 ? 0 : P2 == 8 ? 1 : 2;
   extern __shared__ __attribute__((aligned(16))) uint16_t sm_lds[];
   uint16_t* k_s = sm_lds;                       // [MAPS][KT * DK]
   uint16_t* v_s = sm_lds + MAPS * KT * DK;      // [DV * KT]
@@ -293,7 +299,7 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
   auto fetch = [&](int t) {
     const int64_t blk = P.block_tables[(int64_t)b * P.max_blocks + t];
     const uint16_t* kp = P.kc + (blk * P.G + g) * (int64_t)(MAPS * KT * DK);
-    const uint16_t* vp = P.vc + (blk * P.G + g) * (int64_t)(KT * DV);
+    const uint16_t* vp = P.vc + (blk * P.G + g) * (int64_t)KT * P.v_row;
 #pragma unroll
     for (int m = 0; m < MAPS; ++m)
 #pragma unroll
@@ -303,7 +309,7 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
       const int c = tid + 256 * i;            // block: keys 4 * (c & 15) .. + 3, columns 8 * (c >> 4) .. + 7
       if (c < 2 * DV) {
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) vreg[i][kk] = load8(vp + (int64_t)(4 * (c & 15) + kk) * DV + 8 * (c >> 4));
+        for (int kk = 0; kk < 4; ++kk) vreg[i][kk] = load8(vp + (int64_t)(4 * (c & 15) + kk) * P.v_row + 8 * (c >> 4));
       }
     }
   };
@@ -469,8 +475,21 @@ bool launch_sm_mfma_dv(const SmMfmaParams& P, int dv, dim3 grid, hipStream_t str
   }
 }
 
+// key sizes of a latent plus a rotated part (one map): one value size each
+template <int DK, int DV>
+bool launch_sm_mfma_pair(const SmMfmaParams& P, int dv, dim3 grid, hipStream_t stream) {
+  if (dv != DV) return false;
+  launch_sm_mfma_one<DK, DV, 1>(P, grid, stream);
+  return true;
+}
+
 template <int MAPS>
 bool launch_sm_mfma_dk(const SmMfmaParams& P, int dk, int dv, dim3 grid, hipStream_t stream) {
+  if (MAPS == 1) {
+    if (dk == 96) return launch_sm_mfma_pair<96, 64>(P, dv, grid, stream);
+    if (dk == 192) return launch_sm_mfma_pair<192, 128>(P, dv, grid, stream);
+    if (dk == 320) return launch_sm_mfma_pair<320, 256>(P, dv, grid, stream);
+  }
   switch (dk) {
     case 32: return launch_sm_mfma_dv<32, MAPS>(P, dv, grid, stream);
     case 64: return launch_sm_mfma_dv<64, MAPS>(P, dv, grid, stream);
@@ -496,7 +515,8 @@ template <int DK, int DV, int MAPS>
 __device__ __forceinline__ void softmax_decode_mfma_body(
     float* __restrict__ ws, const uint16_t* __restrict__ q, int64_t q_stride, const uint16_t* __restrict__ kc,
     const uint16_t* __restrict__ vc, const int32_t* __restrict__ block_tables, int max_blocks,
-    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int H, int G, float scale_log2, int window) {
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int H, int G, float scale_log2, int window,
+    int v_row) {
   constexpr int KT = 64;
   constexpr int DS = DK / 32;
   constexpr int DT = DV / 16;
@@ -542,7 +562,7 @@ __device__ __forceinline__ void softmax_decode_mfma_body(
     const bool have = pg <= p_hi;
     const int64_t blk = have ? bt[pg] : 0;
     const uint16_t* kp = kc + (blk * G + g) * (int64_t)(MAPS * KT * DK);
-    const uint16_t* vp = vc + (blk * G + g) * (int64_t)(KT * DV);
+    const uint16_t* vp = vc + (blk * G + g) * (int64_t)KT * v_row;
     __syncthreads();   // the previous page's reads of this wave's tile are done
     if (have) {
       // all of the page's V loads in flight together, then the transposed stores
@@ -551,7 +571,7 @@ __device__ __forceinline__ void softmax_decode_mfma_body(
       for (int bi = 0; bi < VBLK; ++bi) {
         const int c = lane + 64 * bi;            // block: keys 4 * (c & 15) .. + 3, columns 8 * (c >> 4) .. + 7
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) vreg[bi][kk] = load8(vp + (int64_t)(4 * (c & 15) + kk) * DV + 8 * (c >> 4));
+        for (int kk = 0; kk < 4; ++kk) vreg[bi][kk] = load8(vp + (int64_t)(4 * (c & 15) + kk) * v_row + 8 * (c >> 4));
       }
 #pragma unroll
       for (int bi = 0; bi < VBLK; ++bi) {
@@ -707,18 +727,20 @@ template <int DK, int DV, int MAPS>
 __global__ void __launch_bounds__(256) softmax_decode_mfma_kernel(
     float* __restrict__ ws, const uint16_t* __restrict__ q, int64_t q_stride, const uint16_t* __restrict__ kc,
     const uint16_t* __restrict__ vc, const int32_t* __restrict__ block_tables, int max_blocks,
-    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int H, int G, float scale_log2, int window) {
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int H, int G, float scale_log2, int window,
+    int v_row) {
   softmax_decode_mfma_body<DK, DV, MAPS>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2,
-                                         window);
+                                         window, v_row);
 }
 
 template <int DK, int DV, int MAPS>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) softmax_decode_mfma_kernel_w2(
     float* __restrict__ ws, const uint16_t* __restrict__ q, int64_t q_stride, const uint16_t* __restrict__ kc,
     const uint16_t* __restrict__ vc, const int32_t* __restrict__ block_tables, int max_blocks,
-    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int H, int G, float scale_log2, int window) {
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int H, int G, float scale_log2, int window,
+    int v_row) {
   softmax_decode_mfma_body<DK, DV, MAPS>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2,
-                                         window);
+                                         window, v_row);
 }
 
 // one wave per (token row, head): merge the partials of each map, a_0 - lam * a_1, unit RMS, gate
@@ -768,7 +790,7 @@ __global__ void __launch_bounds__(64) softmax_decode_reduce_kernel(
 template <int DK, int DV, int MAPS>
 void launch_sm_decode_one(float* ws, const uint16_t* q, int64_t q_stride, const uint16_t* kc, const uint16_t* vc,
                           const int32_t* block_tables, int max_blocks, const int32_t* tok_seq, const int32_t* pos,
-                          int H, int G, float scale_log2, int window, dim3 grid, hipStream_t stream) {
+                          int H, int G, float scale_log2, int window, int v_row, dim3 grid, hipStream_t stream) {
   constexpr size_t tiles = (size_t)4 * DV * 64 * sizeof(uint16_t);
   constexpr size_t merge = (size_t)(4 * MAPS * 2 * 16 + MAPS * 16 * DV) * sizeof(float);
   constexpr size_t smem = tiles > merge ? tiles : merge;
@@ -781,7 +803,7 @@ void launch_sm_decode_one(float* ws, const uint16_t* q, int64_t q_stride, const 
     }
     softmax_decode_mfma_kernel_w2<DK, DV, MAPS><<<grid, 256, smem, stream>>>(ws, q, q_stride, kc, vc, block_tables,
                                                                             max_blocks, tok_seq, pos, H, G, scale_log2,
-                                                                            window);
+                                                                            window, v_row);
   } else {
     if (smem > 65536 && !attr_set) {
       (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&softmax_decode_mfma_kernel<DK, DV, MAPS>),
@@ -790,15 +812,15 @@ void launch_sm_decode_one(float* ws, const uint16_t* q, int64_t q_stride, const 
     }
     softmax_decode_mfma_kernel<DK, DV, MAPS><<<grid, 256, smem, stream>>>(ws, q, q_stride, kc, vc, block_tables,
                                                                          max_blocks, tok_seq, pos, H, G, scale_log2,
-                                                                         window);
+                                                                         window, v_row);
   }
 }
 
-#define NGA_SM_DEC_ARGS ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, window, grid, stream
+#define NGA_SM_DEC_ARGS ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, window, v_row, grid, stream
 template <int DK, int MAPS>
 bool launch_sm_decode_dv(float* ws, const uint16_t* q, int64_t q_stride, const uint16_t* kc, const uint16_t* vc,
                          const int32_t* block_tables, int max_blocks, const int32_t* tok_seq, const int32_t* pos, int H,
-                         int G, float scale_log2, int window, int dv, dim3 grid, hipStream_t stream) {
+                         int G, float scale_log2, int window, int v_row, int dv, dim3 grid, hipStream_t stream) {
   switch (dv) {
     case 32: launch_sm_decode_one<DK, 32, MAPS>(NGA_SM_DEC_ARGS); return true;
     case 64: launch_sm_decode_one<DK, 64, MAPS>(NGA_SM_DEC_ARGS); return true;
@@ -816,13 +838,18 @@ bool launch_sm_decode_dv(float* ws, const uint16_t* q, int64_t q_stride, const u
 template <int MAPS>
 bool launch_sm_decode_dk(float* ws, const uint16_t* q, int64_t q_stride, const uint16_t* kc, const uint16_t* vc,
                          const int32_t* block_tables, int max_blocks, const int32_t* tok_seq, const int32_t* pos, int H,
-                         int G, float scale_log2, int window, int dk, int dv, dim3 grid, hipStream_t stream) {
-#define NGA_SM_DEC_DV(DKV) launch_sm_decode_dv<DKV, MAPS>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, window, dv, grid, stream)
+                         int G, float scale_log2, int window, int v_row, int dk, int dv, dim3 grid, hipStream_t stream) {
+#define NGA_SM_DEC_DV(DKV) launch_sm_decode_dv<DKV, MAPS>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, window, v_row, dv, grid, stream)
+  if (MAPS == 1) {   // key sizes of a latent plus a rotated part: one value size each
+    if (dk == 96 && dv == 64) { launch_sm_decode_one<96, 64, 1>(NGA_SM_DEC_ARGS); return true; }
+    if (dk == 192 && dv == 128) { launch_sm_decode_one<192, 128, 1>(NGA_SM_DEC_ARGS); return true; }
+    if (dk == 320 && dv == 256) { launch_sm_decode_one<320, 256, 1>(NGA_SM_DEC_ARGS); return true; }
+  }
   switch (dk) {
     case 32: return NGA_SM_DEC_DV(32);
     case 64: return NGA_SM_DEC_DV(64);
     case 128: return NGA_SM_DEC_DV(128);
-    case 256: return MAPS == 1 ? launch_sm_decode_dv<256, 1>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, window, dv, grid, stream) : false;
+    case 256: return MAPS == 1 ? launch_sm_decode_dv<256, 1>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, window, v_row, dv, grid, stream) : false;
     default: return false;
   }
 #undef NGA_SM_DEC_DV
@@ -849,22 +876,27 @@ void launch_softmax_decode_mfma(uint16_t* out, float* ws, int parts, const uint1
                                 const uint16_t* gate, int64_t g_stride, const uint16_t* kc, const uint16_t* vc,
                                 const int32_t* block_tables, int max_blocks, const int32_t* tok_seq,
                                 const int32_t* pos, int64_t T, int H, int G, int dk, int dv, float scale, int window,
-                                int maps, float lam, float unit_eps, float out_scale, hipStream_t stream) {
+                                int maps, float lam, float unit_eps, float out_scale, bool v_in_k,
+                                hipStream_t stream) {
   if (T == 0) return;
   const dim3 grid((unsigned)parts, (unsigned)(G * ((H / G + 15) / 16)), (unsigned)T);
   const float scale_log2 = scale * 1.4426950408889634f;
+  const int v_row = v_in_k ? dk : dv;
   const bool ok = maps == 2 ? launch_sm_decode_dk<2>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G,
-                                                     scale_log2, window, dk, dv, grid, stream)
+                                                     scale_log2, window, v_row, dk, dv, grid, stream)
                             : launch_sm_decode_dk<1>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G,
-                                                     scale_log2, window, dk, dv, grid, stream);
+                                                     scale_log2, window, v_row, dk, dv, grid, stream);
   if (!ok) abort();   // the caller checks softmax_attention_mfma_supported
   softmax_decode_reduce_kernel<<<dim3((unsigned)T, (unsigned)H), 64, 0, stream>>>(out, ws, parts, gate, g_stride, H,
                                                                                    dv, maps, lam, unit_eps, out_scale);
 }
 
-// Head sizes of the MFMA forms: dk, dv in {32, 64, 128} (one map: also 256).
+// Head sizes of the MFMA forms: dk, dv in {32, 64, 128} (one map: also 256, and the pairs
+// (96, 64), (192, 128), (320, 256) of a latent with a rotated key part).
 bool softmax_attention_mfma_supported(int dk, int dv, int group, int maps) {
   auto ok = [&](int d) { return d == 32 || d == 64 || d == 128 || (maps == 1 && d == 256); };
+  if (maps == 1 && group >= 1 && ((dk == 96 && dv == 64) || (dk == 192 && dv == 128) || (dk == 320 && dv == 256)))
+    return true;
   return (maps == 1 || maps == 2) && ok(dk) && ok(dv) && group >= 1;
 }
 
@@ -875,10 +907,10 @@ void launch_softmax_attention_mfma(uint16_t* out, const uint16_t* q, int64_t q_s
                                    const int32_t* block_tables, int max_blocks, const int32_t* cu_q,
                                    const int32_t* ctx_lens, int B, int max_q_len, int H, int G, int dk, int dv,
                                    float scale, int window, int maps, float lam, float unit_eps, float out_scale,
-                                   hipStream_t stream) {
+                                   bool v_in_k, hipStream_t stream) {
   if (B == 0 || max_q_len == 0) return;
   SmMfmaParams P{out, q, gate, kc, vc, block_tables, cu_q, ctx_lens, q_stride, g_stride, max_blocks, H, G, window,
-                 scale * 1.4426950408889634f, lam, unit_eps, out_scale};
+                 scale * 1.4426950408889634f, lam, unit_eps, out_scale, v_in_k ? dk : dv};
   const dim3 grid((unsigned)((max_q_len + 63) / 64), (unsigned)H, (unsigned)B);
   const bool ok = maps == 2 ? launch_sm_mfma_dk<2>(P, dk, dv, grid, stream) : launch_sm_mfma_dk<1>(P, dk, dv, grid, stream);
   if (!ok) abort();   // the caller checks softmax_attention_mfma_supported
@@ -901,20 +933,21 @@ void launch_headnorm_cache(void* proj, int64_t stride, const int32_t* slots, voi
 void launch_softmax_attention(void* out, const void* q, int64_t q_stride, const void* gate, int64_t g_stride,
                               const void* kc, const void* vc, const int32_t* block_tables, int max_blocks,
                               const int32_t* tok_seq, const int32_t* pos, int64_t T, int H, int G, int dk, int dv,
-                              float scale, int window, int maps, float lam, float unit_eps, float out_scale, bool f32,
-                              hipStream_t stream) {
+                              float scale, int window, int maps, float lam, float unit_eps, float out_scale, bool v_in_k,
+                              bool f32, hipStream_t stream) {
   if (T == 0) return;
+  const int v_row = v_in_k ? dk : dv;
   const dim3 grid((unsigned)T, (unsigned)H);
   const size_t smem = (size_t)(maps * dk + 64) * sizeof(float);
   if (f32)
     softmax_attention_kernel<float><<<grid, 64, smem, stream>>>(
         (float*)out, (const float*)q, q_stride, (const float*)gate, g_stride, (const float*)kc, (const float*)vc,
-        block_tables, max_blocks, tok_seq, pos, H, G, dk, dv, scale, window, maps, lam, unit_eps, out_scale);
+        block_tables, max_blocks, tok_seq, pos, H, G, dk, dv, scale, window, maps, lam, unit_eps, out_scale, v_row);
   else
     softmax_attention_kernel<uint16_t><<<grid, 64, smem, stream>>>(
         (uint16_t*)out, (const uint16_t*)q, q_stride, (const uint16_t*)gate, g_stride, (const uint16_t*)kc,
         (const uint16_t*)vc, block_tables, max_blocks, tok_seq, pos, H, G, dk, dv, scale, window, maps, lam, unit_eps,
-        out_scale);
+        out_scale, v_row);
 }
 
 }  // namespace nga

@@ -552,3 +552,225 @@ def biruvik_layers(pattern: Sequence[str], hidden: int, heads: int, kv_heads: in
         blocks.append(BiruvikLayer(t, m, ReluSqMlpSpec(ff) if ff else None))
     return BiruvikConfig(name=name, vocab_size=vocab_size, hidden=hidden, eps=eps, embed_scale=embed_scale,
                          logit_softcap=logit_softcap, blocks=tuple(blocks))
+
+
+# ---------------------------------------------------------------------------------------------
+# Lumepel: pre-norm layers whose mixers are latent attention with a rotated key part.
+@dataclass(frozen=True)
+class RotarySpec:
+    """Rotary positions on the first ``dims`` elements of a vector: pair i turns by
+    ``p * f_i`` at position p, ``f_i = base^(-2i / dims)``. ``interleaved``: pair i is elements
+    (2i, 2i + 1), else (i, i + dims / 2). ``yarn`` = (factor, original, fast, slow) or None: the
+    frequencies of slow pairs are divided by ``factor`` along a linear ramp over the pair index,
+    and cos / sin are multiplied by ``0.1 ln(factor) + 1`` (:func:`ops.rotary_frequencies`)."""
+
+    dims: int
+    base: float
+    interleaved: bool = False
+    yarn: Optional[tuple] = None
+
+
+@dataclass(frozen=True)
+class RotaryLatentAttentionSpec:
+    """Mixers ``latent_attention`` / ``latent_attention_2``: causal softmax attention whose keys
+    and values are linear maps of one RMS-normed latent of ``kv_rank`` elements per token, plus
+    one rotated key part of ``rot_dim`` elements shared by all heads; a query head is ``dim``
+    unrotated and ``rot_dim`` rotated elements. Only the latent and the rotated key part are
+    cached. ``q_rank`` > 0: the query goes through an RMS-normed latent of its own."""
+
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    kv_rank: int
+    scale: float
+    rot: RotarySpec
+    q_rank: int = 0
+
+
+@dataclass(frozen=True)
+class ClampedGluSpec:
+    """down(g * sigmoid(1.702 g) * (u + 1)) with g = min(gate x, limit), u = clamp(up x, +-limit)."""
+
+    ff: int
+    limit: float
+    kind: str = "dense"
+
+
+@dataclass(frozen=True)
+class SigmoidMoeSpec:
+    """``experts`` clamped-GLU experts of which a token uses the ``top`` with the largest
+    ``sigmoid(router x)``; the scores are the weights as they are (not renormalised) and multiply
+    the expert's *input*. ``shared``: an expert every token uses, times ``sigmoid(sg . x)``."""
+
+    experts: int
+    top: int
+    expert: ClampedGluSpec
+    shared: Optional[ClampedGluSpec] = None
+    kind: str = "moe"
+
+
+@dataclass(frozen=True)
+class LumepelLayer:
+    type: str                 # "latent_attention" | "latent_attention_2"
+    mixer: RotaryLatentAttentionSpec
+    mlp: object = None        # ClampedGluSpec | SigmoidMoeSpec | None
+
+
+_LUMEPEL_MIXERS = ("latent_attention", "latent_attention_2")
+
+
+@dataclass(frozen=True)
+class LumepelConfig:
+    """Lumepel: pre-norm layers on an fp32 residual stream (``x += mixer(norm1(x))``,
+    ``x += ff(norm2(x))``), a scaled embedding, scaled and soft-capped logits. Every size and
+    every constant that can differ between models comes from config.json (:meth:`from_dict`)."""
+
+    name: str = "lumepel"
+    vocab_size: int = 512
+    hidden: int = 128
+    eps: float = 1e-5
+    embed_scale: float = 1.0
+    logit_scale: float = 1.0
+    logit_softcap: float = 0.0      # 0: none
+    blocks: tuple = ()
+    max_position: int = 1 << 20     # no position table: only the engine's bookkeeping is bounded
+    arch: str = "lumepel"
+    bos_id: int = 0
+    eos_ids: tuple = ()
+    chat_format: str = "plain"
+
+    @property
+    def layers(self) -> int:
+        return len(self.blocks)
+
+    @property
+    def is_moe(self) -> bool:
+        return any(isinstance(b.mlp, SigmoidMoeSpec) for b in self.blocks)
+
+    @property
+    def experts_per_tok(self) -> int:
+        """Largest top-k of any layer (sizes the engine's routing workspace)."""
+        return max([b.mlp.top for b in self.blocks if isinstance(b.mlp, SigmoidMoeSpec)] or [1])
+
+    @property
+    def num_experts(self) -> int:
+        return max([b.mlp.experts for b in self.blocks if isinstance(b.mlp, SigmoidMoeSpec)] or [0])
+
+    @staticmethod
+    def _glu(d: dict, what: str) -> ClampedGluSpec:
+        s = ClampedGluSpec(ff=int(d["ff"]), limit=float(d["limit"]))
+        if s.ff < 1 or not s.limit > 0:
+            raise ValueError(f"{what}: ff and limit must be positive")
+        return s
+
+    @classmethod
+    def from_dict(cls, d: dict, name: str = "lumepel") -> "LumepelConfig":
+        blocks = []
+        for i, b in enumerate(d["layers"]):
+            t, m = b["type"], b["mixer"]
+            if t not in _LUMEPEL_MIXERS:
+                raise ValueError(f"layer {i}: unknown mixer type {t!r} (known: {_LUMEPEL_MIXERS})")
+            r = m["rot"]
+            sc = r.get("scaling")
+            rot = RotarySpec(dims=int(r["dims"]), base=float(r["base"]), interleaved=t == "latent_attention",
+                             yarn=None if not sc else (float(sc["factor"]), float(sc["original"]),
+                                                       float(sc["fast"]), float(sc["slow"])))
+            mixer = RotaryLatentAttentionSpec(heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]),
+                                              vdim=int(m["vdim"]), kv_rank=int(m["kv_rank"]), scale=float(m["scale"]),
+                                              rot=rot, q_rank=int(m["q_rank"]) if t == "latent_attention" else 0)
+            if rot.dims % 2 or not 0 < rot.dims <= mixer.rot_dim:
+                raise ValueError(f"layer {i}: rot.dims must be even and at most rot_dim")
+            if t == "latent_attention" and mixer.q_rank < 1:
+                raise ValueError(f"layer {i}: latent_attention needs q_rank")
+            mlp = b.get("mlp")
+            if mlp is not None:
+                kind = mlp.get("kind", "dense")
+                if kind == "dense":
+                    mlp = cls._glu(mlp, f"layer {i} feed-forward")
+                elif kind == "moe":
+                    sh = mlp.get("shared")
+                    mlp = SigmoidMoeSpec(experts=int(mlp["router"]["experts"]), top=int(mlp["router"]["top"]),
+                                         expert=cls._glu(mlp["expert"], f"layer {i} experts"),
+                                         shared=None if not sh else cls._glu(sh, f"layer {i} shared expert"))
+                    if not 1 <= mlp.top <= mlp.experts:
+                        raise ValueError(f"layer {i}: top {mlp.top} of {mlp.experts} experts")
+                else:
+                    raise ValueError(f"layer {i}: unknown feed-forward kind {kind!r}")
+            blocks.append(LumepelLayer(type=t, mixer=mixer, mlp=mlp))
+        return cls(name=name, vocab_size=int(d["vocab"]), hidden=int(d["width"]), eps=float(d["norm"]["eps"]),
+                   embed_scale=float(d["embedding"]["scale"]), logit_scale=float(d.get("logit_scale", 1.0)),
+                   logit_softcap=float(d.get("logit_softcap") or 0.0), blocks=tuple(blocks))
+
+    def to_json_dict(self) -> dict:
+        """The config.json form (inverse of :meth:`from_dict`)."""
+        layers = []
+        for b in self.blocks:
+            m = b.mixer
+            rot = {"base": m.rot.base, "dims": m.rot.dims}
+            if m.rot.yarn:
+                rot["scaling"] = dict(zip(("factor", "original", "fast", "slow"), m.rot.yarn))
+            mx = {"heads": m.heads, "dim": m.dim, "rot_dim": m.rot_dim, "vdim": m.vdim, "kv_rank": m.kv_rank,
+                  "scale": m.scale, "rot": rot}
+            if b.type == "latent_attention":
+                mx["q_rank"] = m.q_rank
+            f = b.mlp
+            if isinstance(f, SigmoidMoeSpec):
+                ff = {"kind": "moe", "router": {"experts": f.experts, "top": f.top},
+                      "expert": {"ff": f.expert.ff, "limit": f.expert.limit}}
+                if f.shared is not None:
+                    ff["shared"] = {"ff": f.shared.ff, "limit": f.shared.limit}
+            elif f is not None:
+                ff = {"kind": "dense", "ff": f.ff, "limit": f.limit}
+            else:
+                ff = None
+            layers.append({"type": b.type, "mixer": mx, "mlp": ff})
+        return {"architecture": "Lumepel", "vocab": self.vocab_size, "width": self.hidden,
+                "embedding": {"scale": self.embed_scale}, "norm": {"eps": self.eps},
+                "logit_scale": self.logit_scale, "logit_softcap": self.logit_softcap, "layers": layers}
+
+    def num_params(self) -> int:
+        H = self.hidden
+        n = 2 * self.vocab_size * H + H
+        for b in self.blocks:
+            m = b.mixer
+            nq = m.heads * (m.dim + m.rot_dim)
+            n += H + (H * m.q_rank + m.q_rank + m.q_rank * nq if m.q_rank else H * nq)
+            n += H * (m.kv_rank + m.rot_dim) + m.kv_rank + m.kv_rank * m.heads * (m.dim + m.vdim) + H * m.heads * m.vdim
+            f = b.mlp
+            if isinstance(f, SigmoidMoeSpec):
+                n += H + f.experts * (3 * H * f.expert.ff + H)
+                if f.shared is not None:
+                    n += 3 * H * f.shared.ff + H
+            elif f is not None:
+                n += H + 3 * H * f.ff
+        return n
+
+    def to_dict(self):
+        return asdict(self)
+
+
+def lumepel_layers(pattern: Sequence[str], hidden: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int,
+                   q_rank: int, ff: int, experts: int = 0, top: int = 2, expert_ff: int = 0, shared_ff: int = 0,
+                   limit: float = 7.0, rot_base: float = 10000.0, yarn: Optional[tuple] = None,
+                   vocab_size: int = 32768, embed_scale: float = 1.0, logit_scale: float = 1.0,
+                   logit_softcap: float = 30.0, eps: float = 1e-5, name: str = "lumepel") -> LumepelConfig:
+    """A Lumepel config from a pattern of mixer types with the same sizes in every layer
+    (benchmarks, tests). ``experts`` > 0: every feed-forward is a mixture of ``experts`` experts of
+    ``expert_ff`` (plus a shared one of ``shared_ff``), else dense of ``ff`` (0: none)."""
+    blocks = []
+    for t in pattern:
+        if t not in _LUMEPEL_MIXERS:
+            raise ValueError(f"unknown mixer type {t!r}")
+        lat = t == "latent_attention"
+        rot = RotarySpec(rot_dim, rot_base, interleaved=lat, yarn=yarn if lat else None)
+        m = RotaryLatentAttentionSpec(heads, dim, rot_dim, vdim, kv_rank, (dim + rot_dim) ** -0.5, rot,
+                                      q_rank if lat else 0)
+        if experts:
+            mlp = SigmoidMoeSpec(experts, top, ClampedGluSpec(expert_ff, limit),
+                                 ClampedGluSpec(shared_ff, limit) if shared_ff else None)
+        else:
+            mlp = ClampedGluSpec(ff, limit) if ff else None
+        blocks.append(LumepelLayer(t, m, mlp))
+    return LumepelConfig(name=name, vocab_size=vocab_size, hidden=hidden, eps=eps, embed_scale=embed_scale,
+                         logit_scale=logit_scale, logit_softcap=logit_softcap, blocks=tuple(blocks))

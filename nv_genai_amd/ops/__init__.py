@@ -498,7 +498,7 @@ def softcap_(z: torch.Tensor, cap: float) -> torch.Tensor:
     """fp32 logits in place: ``cap * tanh(z / cap)``."""
     if not _gpu(z):
         return ref.softcap_(z, cap)
-    kernels().softcap(z, float(cap))
+    kernels().softcap(z, float(cap), 1.0)
     return z
 
 
@@ -531,7 +531,7 @@ def headnorm_cache_(proj, slots, kc, vc, nq: int, nk: int, dk: int, nv: int, dv:
 
 def softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H: int, G: int, dk: int, dv: int, scale: float,
                       window: int = 0, maps: int = 1, lam: float = 0.0, unit_eps: Optional[float] = None,
-                      out_scale: float = 1.0, gate=None, out=None):
+                      out_scale: float = 1.0, gate=None, out=None, v_in_k: bool = False):
     """Softmax attention of token rows (prompt portions and single-token rows alike) over row-
     major pages K [blocks, G * maps, 64, dk], V [blocks, G, 64, dv]. The query at position i
     sees keys ``j <= i`` (``window`` > 0: and ``i - j < window``). ``maps`` (1 or 2) score maps per
@@ -541,21 +541,25 @@ def softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H: int, G: int, dk:
     root mean square (eps inside the root) and multiply by ``out_scale``. ``gate`` [T, H]: the
     head outputs are multiplied by ``sigmoid(gate)``. ``tok_seq[t]`` is the block-table row of
     token t, ``pos[t]`` its position (negative: padding row, zeros out). Scores, softmax and
-    accumulation are fp32."""
+    accumulation are fp32. ``v_in_k`` (one map, dv <= dk): the values are the first dv elements of
+    the key rows (``vc`` is not read) - keys with extra key-only columns behind a shared latent."""
+    if v_in_k and (maps != 1 or dv > dk):
+        raise ValueError("values inside the key rows: one map and dv <= dk")
     if not _gpu(q):
         return ref.softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv, scale, window, maps, lam,
-                                     unit_eps, out_scale, gate)
+                                     unit_eps, out_scale, gate, v_in_k)
     if out is None:
         out = torch.empty(q.shape[0], H * dv, dtype=q.dtype, device=q.device)
-    kernels().softmax_attention(out, q, gate, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv, float(scale),
-                                int(window), int(maps), float(lam), -1.0 if unit_eps is None else float(unit_eps),
-                                float(out_scale))
+    kernels().softmax_attention(out, q, gate, kc, kc if v_in_k else vc, block_tables, tok_seq, pos, H, G, dk, dv,
+                                float(scale), int(window), int(maps), float(lam),
+                                -1.0 if unit_eps is None else float(unit_eps), float(out_scale), bool(v_in_k))
     return out
 
 
 def softmax_attention_mfma_ok(q: torch.Tensor, dk: int, dv: int, group: int = 1, maps: int = 1) -> bool:
     """The MFMA softmax attention kernels take bf16 GPU rows (16-byte aligned) with dk, dv in
-    {32, 64, 128} (one map: also 256)."""
+    {32, 64, 128} (one map: also 256, and the key sizes 96 / 192 / 320 of a latent with a rotated
+    part)."""
     return (_gpu(q) and q.dtype == torch.bfloat16 and have_kernels() and q.stride(0) % 8 == 0
             and q.data_ptr() % 16 == 0
             and bool(kernels().softmax_attention_mfma_supported(int(dk), int(dv), int(group), int(maps))))
@@ -571,25 +575,29 @@ def _rows_of_portions(cu_q, ctx_lens, T: int, dev):
 
 def softmax_attention_prefill(q, kc, vc, block_tables, cu_q, ctx_lens, max_q_len: int, H: int, G: int, dk: int,
                               dv: int, scale: float, window: int = 0, maps: int = 1, lam: float = 0.0,
-                              unit_eps: Optional[float] = None, out_scale: float = 1.0, gate=None, out=None):
+                              unit_eps: Optional[float] = None, out_scale: float = 1.0, gate=None, out=None,
+                              v_in_k: bool = False):
     """:func:`softmax_attention` of prompt portions on MFMA tiles: sequence b owns token rows
     ``[cu_q[b], cu_q[b + 1])``, the last ones of its ``ctx_lens[b]`` keys. Rows the tile kernel
     does not take (fp32, other head sizes, CPU) run the row form."""
     if not softmax_attention_mfma_ok(q, dk, dv, H // G, maps):
         seq, pos = _rows_of_portions(cu_q, ctx_lens, q.shape[0], q.device)
         return softmax_attention(q, kc, vc, block_tables, seq, pos, H, G, dk, dv, scale, window, maps, lam, unit_eps,
-                                 out_scale, gate, out=out)
+                                 out_scale, gate, out=out, v_in_k=v_in_k)
+    if v_in_k and (maps != 1 or dv > dk):
+        raise ValueError("values inside the key rows: one map and dv <= dk")
     if out is None:
         out = torch.empty(q.shape[0], H * dv, dtype=q.dtype, device=q.device)
-    kernels().softmax_attention_prefill(out, q, gate, kc, vc, block_tables, cu_q, ctx_lens, int(max_q_len), H, G, dk,
-                                        dv, float(scale), int(window), int(maps), float(lam),
-                                        -1.0 if unit_eps is None else float(unit_eps), float(out_scale))
+    kernels().softmax_attention_prefill(out, q, gate, kc, kc if v_in_k else vc, block_tables, cu_q, ctx_lens,
+                                        int(max_q_len), H, G, dk, dv, float(scale), int(window), int(maps), float(lam),
+                                        -1.0 if unit_eps is None else float(unit_eps), float(out_scale), bool(v_in_k))
     return out
 
 
 def softmax_attention_rows(q, kc, vc, block_tables, tok_seq, pos, H: int, G: int, dk: int, dv: int, scale: float,
                            max_ctx: int, window: int = 0, maps: int = 1, lam: float = 0.0,
-                           unit_eps: Optional[float] = None, out_scale: float = 1.0, gate=None, out=None):
+                           unit_eps: Optional[float] = None, out_scale: float = 1.0, gate=None, out=None,
+                           v_in_k: bool = False):
     """:func:`softmax_attention` of single-token rows (decode rows; any rows work) on the page-
     parallel MFMA kernel: the query heads that share a KV head are the columns of one tile, so a
     page is read once per group; the visible pages of a row are split over several workgroups
@@ -597,17 +605,112 @@ def softmax_attention_rows(q, kc, vc, block_tables, tok_seq, pos, H: int, G: int
     normalises and gates. ``max_ctx`` bounds the rows' positions (launch shape)."""
     if not softmax_attention_mfma_ok(q, dk, dv, H // G, maps):
         return softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv, scale, window, maps, lam,
-                                 unit_eps, out_scale, gate, out=out)
+                                 unit_eps, out_scale, gate, out=out, v_in_k=v_in_k)
+    if v_in_k and (maps != 1 or dv > dk):
+        raise ValueError("values inside the key rows: one map and dv <= dk")
     C = kernels()
     T = q.shape[0]
     parts = int(C.softmax_decode_parts(max(T, 1), G * -(-(H // G) // 16), int(max_ctx), int(window)))
     ws = torch.empty(T * H * maps * parts * (dv + 4), dtype=torch.float32, device=q.device)
     if out is None:
         out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
-    C.softmax_attention_decode(out, ws, parts, q, gate, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv,
-                               float(scale), int(window), int(maps), float(lam),
-                               -1.0 if unit_eps is None else float(unit_eps), float(out_scale))
+    C.softmax_attention_decode(out, ws, parts, q, gate, kc, kc if v_in_k else vc, block_tables, tok_seq, pos, H, G, dk,
+                               dv, float(scale), int(window), int(maps), float(lam),
+                               -1.0 if unit_eps is None else float(unit_eps), float(out_scale), bool(v_in_k))
     return out
+
+
+# ------------------------------------------------------------------------- pre-norm fp32 stream, rotated latent attention
+def residual_add_rmsnorm_(x: torch.Tensor, y: torch.Tensor, w: Optional[torch.Tensor], eps: float,
+                          dtype: torch.dtype) -> Optional[torch.Tensor]:
+    """Pre-norm step on an fp32 stream: ``x += y`` in place (fp32 sum), and returns
+    ``rmsnorm(x) * w`` (the next sub-layer's input) in ``dtype`` from the same launch. ``w`` None:
+    the sum only, returns None."""
+    out = None if w is None else torch.empty(x.shape, dtype=dtype, device=x.device)
+    if not _gpu(x):
+        ref.residual_add_rmsnorm_(x, y, w, eps, out)
+        return out
+    kernels().residual_add_rmsnorm(x, y, w, float(eps), out)
+    return out
+
+
+def rotary_frequencies(dims: int, base: float, yarn=None) -> Tuple[torch.Tensor, float]:
+    """(float64 frequencies [dims / 2], factor on cos and sin) of rotary positions on ``dims``
+    elements: ``f_i = base^(-2i / dims)``. ``yarn`` = (factor, original, fast, slow): with
+    ``pair(t) = dims ln(original / (2 pi t)) / (2 ln base)`` the index of the pair that turns t
+    times in ``original`` positions, ``lo = max(floor(pair(fast)), 0)``,
+    ``hi = min(ceil(pair(slow)), dims - 1)`` and ``ramp_i = clamp((i - lo) / max(hi - lo, 0.001),
+    0, 1)``, the frequency is ``f_i / factor * ramp_i + f_i (1 - ramp_i)`` and cos / sin are
+    multiplied by ``0.1 ln(factor) + 1``."""
+    import math
+
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = torch.tensor([float(base) ** (-2.0 * k / dims) for k in range(dims // 2)], dtype=torch.float64)
+    if not yarn:
+        return f, 1.0
+    factor, orig, fast, slow = (float(v) for v in yarn)
+
+    def pair(t):
+        return dims * math.log(orig / (2.0 * math.pi * t)) / (2.0 * math.log(float(base)))
+
+    lo, hi = max(math.floor(pair(fast)), 0), min(math.ceil(pair(slow)), dims - 1)
+    ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+    return f / factor * ramp + f * (1.0 - ramp), 0.1 * math.log(factor) + 1.0
+
+
+def latent_rope_cache_(proj, pos, slots, page, freq, mag: float, interleaved: bool, rot_dims: int, rot_dim: int,
+                       eps: float, kv=None, q=None, q_out=None, norm=None):
+    """Projection rows of latent attention with a rotated key part, in one launch per row:
+
+    * ``norm`` = (column, n, weight): RMS-normalise ``proj[:, column : column + n]`` in place (a
+      query latent in front of its up-projection);
+    * ``kv`` = (column, r, weight): ``proj[:, column : column + r]`` RMS-normalised (the latent)
+      and the ``rot_dim`` columns behind it with rotary positions (the key part all heads share)
+      go into the token's page slot, ``page`` [blocks, 1, 64, r + rot_dim] (``slots`` < 0: no
+      write);
+    * ``q`` = (column, heads, dim): heads of [dim | rot_dim] columns; the rotated parts get rotary
+      positions and are written behind the first ``W - rot_dim`` columns of every head of
+      ``q_out`` [T, heads * W] (those columns are left for the folded unrotated part).
+
+    Rotary positions: on the first ``rot_dims`` elements of a rotated part, pair i at angle
+    ``pos * freq[i]`` (float64 product, reduced to one turn before the fp32 cos / sin), cos and
+    sin times ``mag``; pairs are (2i, 2i + 1) when ``interleaved``, else (i, i + rot_dims / 2).
+    Norms and rotations are fp32."""
+    if rot_dims % 2 or rot_dims > rot_dim or freq.numel() != rot_dims // 2:
+        raise ValueError("rotary positions: an even number of elements, at most the rotated part")
+    if q is not None and (q_out is None or q_out.shape[1] % q[1] or q_out.shape[1] // q[1] < rot_dim):
+        raise ValueError("q_out must hold heads * W columns with W >= rot_dim")
+    if not _gpu(proj):
+        return ref.latent_rope_cache_(proj, pos, slots, page, freq, mag, interleaved, rot_dims, rot_dim, eps, kv, q,
+                                      q_out, norm)
+    n_off, n_n, n_w = norm if norm is not None else (-1, 0, None)
+    k_off, k_r, k_w = kv if kv is not None else (-1, 0, None)
+    q_off, q_h, q_d = q if q is not None else (-1, 0, 0)
+    kernels().latent_rope_cache(proj, pos, slots, page if kv is not None else None, freq, float(mag),
+                                bool(interleaved), int(rot_dims), int(rot_dim), float(eps), int(k_off), int(k_r), k_w,
+                                int(q_off), int(q_h), int(q_d), q_out, int(n_off), int(n_n), n_w)
+    return proj
+
+
+def clamped_glu(x: torch.Tensor, F: int, limit: float, alpha: float = 1.702, gate_col: int = -1) -> torch.Tensor:
+    """Rows ``[gate F | up F | ...]`` -> ``g * sigmoid(alpha g) * (u + 1)`` [T, F] with
+    ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``; ``gate_col`` >= 0: times
+    ``sigmoid(x[:, gate_col])`` (one gate per row). fp32 math, bf16 or fp32 rows, any F."""
+    if not _gpu(x):
+        return ref.clamped_glu(x, F, limit, alpha, gate_col)
+    out = torch.empty(x.shape[0], F, dtype=x.dtype, device=x.device)
+    kernels().clamped_glu(out, x, int(F), float(limit), float(alpha), int(gate_col))
+    return out
+
+
+def scale_softcap_(z: torch.Tensor, scale: float, cap: float) -> torch.Tensor:
+    """fp32 logits in place: ``z * scale``, then ``cap * tanh(z / cap)`` when ``cap`` > 0."""
+    if cap > 0:
+        if not _gpu(z):
+            return ref.softcap_(z.mul_(scale), cap)
+        kernels().softcap(z, float(cap), float(scale))
+        return z
+    return z.mul_(scale) if scale != 1.0 else z
 
 
 # ------------------------------------------------------------------------- gated linear recurrence
@@ -911,10 +1014,84 @@ def moe_ffn(x: torch.Tensor, router: torch.Tensor, w13: torch.Tensor, w2: torch.
                 ws.tiles, mt)
     h = torch.empty(M, F, dtype=x.dtype, device=x.device)
     C.moe_gemm(x, w13, ws.sorted_tok, ws.sorted_w, ws.tiles, mt, bm, h, 0,
-               0 if act == "silu" else 1)
+               0 if act == "silu" else 1, 0.0, 0.0, False)
     y = torch.empty(M, H, dtype=x.dtype, device=x.device)
-    C.moe_gemm(h, w2, ws.sorted_tok, ws.sorted_w, ws.tiles, mt, bm, y, 1, 0)
+    C.moe_gemm(h, w2, ws.sorted_tok, ws.sorted_w, ws.tiles, mt, bm, y, 1, 0, 0.0, 0.0, False)
     C.moe_combine(y, ws.inv, T, int(k), out)
+    return out
+
+
+def moe_route_scores(logits: torch.Tensor, k: int, score: str = "sigmoid", renorm: bool = False,
+                     ws: Optional["MoEWorkspace"] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Routing from fp32 logits [T, E]: the ``k`` experts with the largest score per row (ties: the
+    lower index), ids int32 [T, k] and fp32 weights [T, k] = ``sigmoid(logit)`` or the softmax
+    probability, as they are or renormalised over the k (``renorm``)."""
+    if score not in ("sigmoid", "softmax"):
+        raise ValueError(f"unknown score {score!r}")
+    if logits.dtype != torch.float32:
+        raise ValueError("router logits are fp32")
+    if not _gpu(logits):
+        return ref.moe_route_scores(logits, k, score, renorm)
+    T, E = logits.shape
+    if ws is not None and ws.rows * ws.k >= T * k:
+        ids, w = ws.ids[:T * k].view(T, k), ws.w[:T * k].view(T, k)
+    else:
+        ids = torch.empty(T, k, dtype=torch.int32, device=logits.device)
+        w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+    kernels().moe_route_scores(logits, int(k), 0 if score == "sigmoid" else 1, bool(renorm), ids, w)
+    return ids, w
+
+
+def moe_mfma_ok(x: torch.Tensor, F: int) -> bool:
+    """The grouped MFMA GEMMs take bf16 rows with width % 256 == 0 and expert ff % 128 == 0."""
+    return _gpu(x) and x.dtype == torch.bfloat16 and x.shape[1] % 256 == 0 and F % 128 == 0
+
+
+def moe_glu_experts(x: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor,
+                    limit: float, alpha: float = 1.702, weight_input: bool = True, add: Optional[torch.Tensor] = None,
+                    ws: Optional["MoEWorkspace"] = None) -> torch.Tensor:
+    """Routed clamped-GLU experts on rows x [T, H] -> [T, H]: the sum over a row's experts
+    (``ids`` / ``wts`` [T, k] from :func:`moe_route_scores`) of
+    ``down_e(g * sigmoid(alpha g) * (u + 1))``, ``g = min(gate_e(s x), limit)``,
+    ``u = clamp(up_e(s x), -limit, limit)`` with the routing weight on the expert's input
+    (``weight_input``; else ``s = 1`` and the weight multiplies the expert's output). ``w13``
+    [E, 2F, H] = [gate | up] rows per expert, ``w2`` [E, H, F]. ``add`` [T, H]: added to the sum in
+    the combining kernel (a shared expert's output).
+
+    GPU: ``moe_align`` (tokens sorted by expert, M-tile table) -> grouped gate|up GEMM with the
+    weight and the activation in its epilogue -> grouped down GEMM -> combine (fp32 sum per token).
+    bf16 rows with MFMA-sized experts run the grouped MFMA GEMMs, everything else (fp32, other
+    sizes) a tiled fp32-accumulating kernel of the same structure."""
+    if not _gpu(x):
+        return ref.moe_glu_experts(x, ids, wts, w13, w2, limit, alpha, weight_input, add)
+    C = kernels()
+    T, H = x.shape
+    E, F2, K = w13.shape
+    F, k = F2 // 2, ids.shape[1]
+    out = torch.empty(T, H, dtype=x.dtype, device=x.device)
+    if T == 0:
+        return out
+    M = T * k
+    if ws is None:
+        ws = MoEWorkspace.get(T, k, E, x.device)
+    if ws.rows * ws.k < M or ws.E < E:
+        raise ValueError(f"MoE workspace for {ws.rows} rows x top-{ws.k} / {ws.E} experts cannot take "
+                         f"{T} rows x top-{k} / {E} experts")
+    mfma = moe_mfma_ok(x, F)
+    bm = 64 if (not mfma or M <= 256 * E) else 128
+    mt = -(-M // bm) + E
+    C.moe_align(ids.reshape(-1), wts.reshape(-1), T, int(k), 0, E, bm, ws.sorted_tok, ws.sorted_w, ws.inv, ws.tiles, mt)
+    h = torch.empty(M, F, dtype=x.dtype, device=x.device)
+    y = torch.empty(M, H, dtype=x.dtype, device=x.device)
+    if mfma:
+        C.moe_gemm(x, w13, ws.sorted_tok, ws.sorted_w, ws.tiles, mt, bm, h, 0, 2, float(limit), float(alpha),
+                   bool(weight_input))
+        C.moe_gemm(h, w2, ws.sorted_tok, ws.sorted_w, ws.tiles, mt, bm, y, 1, 0, 0.0, 0.0, bool(weight_input))
+    else:
+        C.moe_gemm_rows(x, w13, ws.sorted_tok, ws.sorted_w, ws.tiles, mt, h, 0, float(limit), float(alpha),
+                        bool(weight_input))
+        C.moe_gemm_rows(h, w2, ws.sorted_tok, ws.sorted_w, ws.tiles, mt, y, 1, 0.0, 0.0, not weight_input)
+    C.moe_combine_rows(y, ws.inv, T, int(k), add, out)
     return out
 
 

@@ -578,11 +578,12 @@ def headnorm_cache_(proj, slots, kc, vc, nq, nk, dk, nv, dv, eps, q_w=None, k_w=
 
 
 def softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv, scale, window=0, maps=1, lam=0.0,
-                      unit_eps=None, out_scale=1.0, gate=None):
+                      unit_eps=None, out_scale=1.0, gate=None, v_in_k=False):
     """Softmax attention of token rows over row-major pages, one row at a time. ``maps`` score
     maps per head (q head (h, m) at column (h * maps + m) * dk, k head (h // (H / G)) * maps + m,
     v head h // (H / G)), combined as a_0 - lam * a_1; optional unit RMS per head (times
-    ``out_scale``) and a per-head sigmoid gate."""
+    ``out_scale``) and a per-head sigmoid gate. ``v_in_k``: the values are the first dv elements
+    of the key rows."""
     T = q.shape[0]
     out = torch.zeros(T, H, dv, dtype=torch.float32, device=q.device)
     BS = kc.shape[2]
@@ -598,7 +599,7 @@ def softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv, scale
         j = torch.arange(lo, i + 1, device=q.device)
         blk, off = bt[j // BS].long(), j % BS
         k = kc[blk, :, off, :].float().view(-1, G, maps, dk)[:, vh]     # [n, H, maps, dk]
-        v = vc[blk, :, off, :].float()[:, vh]                          # [n, H, dv]
+        v = (kc[blk, :, off, :dv] if v_in_k else vc[blk, :, off, :]).float()[:, vh]   # [n, H, dv]
         s = torch.einsum("hmd,nhmd->hmn", qf[t], k) * scale
         a = torch.einsum("hmn,nhd->hmd", torch.softmax(s, -1), v)
         out[t] = a[:, 0] - lam * a[:, 1] if maps == 2 else a[:, 0]
@@ -645,3 +646,109 @@ def group_rmsnorm(x, w, groups, eps, dtype):
     T = x.shape[0]
     xg = x.view(T, groups, -1)
     return (xg * torch.rsqrt(xg.pow(2).mean(-1, keepdim=True) + eps) * w).reshape(T, -1).to(dtype)
+
+
+# ------------------------------------------------------------------------- pre-norm fp32 stream, rotated latent
+# attention, clamped GLU, sigmoid-routed experts
+def residual_add_rmsnorm_(x, y, w, eps, out):
+    """x (fp32, in place) += y, then out = rmsnorm(x) * w (``w`` None: the sum only)."""
+    x.add_(y.float())
+    if w is not None:
+        out.copy_(x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w)
+    return x
+
+
+def rotary_cos_sin(pos, freq, mag):
+    """(cos, sin) [T, pairs] fp32 of angles pos * freq taken in float64, times ``mag``."""
+    a = pos.to(torch.float64)[:, None] * freq.to(torch.float64)[None, :]
+    return (torch.cos(a) * mag).float(), (torch.sin(a) * mag).float()
+
+
+def _rotate(v, cos, sin, n, interleaved):
+    """Rotary pairs on the first n elements of the last axis of fp32 ``v`` [T, ..., d]."""
+    shape = [v.shape[0]] + [1] * (v.dim() - 2) + [n // 2]
+    c, s = cos.view(shape), sin.view(shape)
+    out = v.clone()
+    if interleaved:
+        a, b = v[..., 0:n:2], v[..., 1:n:2]
+        out[..., 0:n:2] = a * c - b * s
+        out[..., 1:n:2] = b * c + a * s
+    else:
+        a, b = v[..., : n // 2], v[..., n // 2:n]
+        out[..., : n // 2] = a * c - b * s
+        out[..., n // 2:n] = b * c + a * s
+    return out
+
+
+def latent_rope_cache_(proj, pos, slots, page, freq, mag, interleaved, rot_dims, rot_dim, eps, kv=None, q=None,
+                       q_out=None, norm=None):
+    """See :func:`nv_genai_amd.ops.latent_rope_cache_`."""
+    T = proj.shape[0]
+    cos, sin = rotary_cos_sin(pos.clamp(min=0), freq, mag)
+    if norm is not None:
+        off, n, w = norm
+        v = proj[:, off:off + n].float()
+        proj[:, off:off + n] = (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w).to(proj.dtype)
+    if kv is not None:
+        off, r, w = kv
+        c = proj[:, off:off + r].float()
+        c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * w
+        kr = _rotate(proj[:, off + r:off + r + rot_dim].float(), cos, sin, rot_dims, interleaved)
+        sl = slots.long()
+        ok = sl >= 0
+        BS = page.shape[2]
+        page[sl[ok] // BS, 0, sl[ok] % BS, :] = torch.cat([c, kr], 1)[ok].to(page.dtype)
+    if q is not None:
+        off, H, d = q
+        qd = d + rot_dim
+        qr = _rotate(proj[:, off:off + H * qd].float().view(T, H, qd)[:, :, d:], cos, sin, rot_dims, interleaved)
+        w_out = q_out.shape[1] // H
+        q_out.view(T, H, w_out)[:, :, w_out - rot_dim:] = qr.to(q_out.dtype)
+    return proj
+
+
+def clamped_glu(x, F, limit, alpha, gate_col=-1):
+    """Rows [gate F | up F | ...] -> g * sigmoid(alpha g) * (u + 1), g = min(gate, limit),
+    u = clamp(up, +-limit); times sigmoid(x[:, gate_col]) when gate_col >= 0."""
+    xf = x.float()
+    g = xf[:, :F].clamp(max=limit)
+    u = xf[:, F:2 * F].clamp(min=-limit, max=limit)
+    y = g * torch.sigmoid(alpha * g) * (u + 1.0)
+    if gate_col >= 0:
+        y = y * torch.sigmoid(xf[:, gate_col:gate_col + 1])
+    return y.to(x.dtype)
+
+
+def moe_route_scores(logits, k, score="sigmoid", renorm=False):
+    """(ids int32 [T, k], weights fp32 [T, k]): the k largest ``score(logits)`` per row in
+    descending order (ties: the lower expert index first), renormalised over the k or as they are."""
+    lf = logits.float()
+    s = torch.sigmoid(lf) if score == "sigmoid" else torch.softmax(lf, -1)
+    # the activation is monotonic: choose by the logits (exact ties cannot flip through rounding)
+    _, ids = torch.sort(lf, dim=-1, descending=True, stable=True)
+    ids = ids[:, :k]
+    w = torch.gather(s, 1, ids)
+    if renorm:
+        w = w / w.sum(-1, keepdim=True)
+    return ids.to(torch.int32), w
+
+
+def moe_glu_experts(x, ids, wts, w13, w2, limit, alpha, weight_input=True, add=None):
+    """Sum over a row's experts e of expert_e(x) with the routing weight on the expert's input
+    (``weight_input``) or on its output; expert = clamped GLU, ``w13`` [E, 2F, H] = [gate | up],
+    ``w2`` [E, H, F]. ``add`` [T, H] is added to the sum."""
+    E, F2, _ = w13.shape
+    F = F2 // 2
+    out = torch.zeros(x.shape[0], w2.shape[1], dtype=torch.float32, device=x.device)
+    for e in range(E):
+        tok, slot = torch.where(ids == e)
+        if tok.numel() == 0:
+            continue
+        wt = wts[tok, slot].unsqueeze(1)
+        gu = (x[tok].float() @ w13[e].float().t()) * (wt if weight_input else 1.0)
+        h = clamped_glu(gu, F, limit, alpha).to(x.dtype)
+        y = h.float() @ w2[e].float().t()
+        out.index_add_(0, tok, y if weight_input else y * wt)
+    if add is not None:
+        out = out + add.float()
+    return out.to(x.dtype)
