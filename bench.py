@@ -107,7 +107,8 @@ def parse(argv=None):
     ap.add_argument("--design-sizes", default=None,
                     help="--workload designs: comma list of s, m, l (benchmarks/design_compare.py)")
     ap.add_argument("--design-models", default="bidasun",
-                    help="--workload designs: comma list of the designs to run beside Mistral (bidasun, biruvik)")
+                    help="--workload designs: comma list of the designs to run beside the closest Llama-layout model "
+                         "(bidasun, biruvik, lumepel)")
     ap.add_argument("--workload", choices=("rag", "agent", "designs"), default="rag",
                     help="agent: query-decomposition agent, one TP=N replica + N-way sharded index")
     ap.add_argument("--kv-cache-fraction", type=float, default=None)

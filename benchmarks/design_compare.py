@@ -1,8 +1,9 @@
-"""The layer-list designs (Bidasun, Biruvik) beside the closest Llama-layout model (Mistral with a
-sliding window) at equal sizes: prefill and decode throughput through the serving engine, and the
-mixer kernels alone with their distance from the roofline. Random weights, synthetic token ids.
+"""The layer-list designs (Bidasun, Biruvik, Lumepel) beside the closest Llama-layout model at equal
+sizes (Mistral with a sliding window; Mixtral for Lumepel, whose feed-forwards are routed experts):
+prefill and decode throughput through the serving engine, and the design's kernels alone with
+their distance from the roofline. Random weights, synthetic token ids.
 
-    python bench.py --workload designs [--design-sizes s,m,l] [--design-models bidasun,biruvik]
+    python bench.py --workload designs [--design-sizes s,m,l] [--design-models bidasun,biruvik,lumepel]
 
 Prints one JSON line (``metric: design_compare``); bench.py's default workload is untouched.
 """
@@ -26,13 +27,30 @@ PEAK_TRANS = 256 * 16 * 2.4e9   # transcendental lanes/s: 256 CUs x 4 SIMDs x 4 
 PEAK_VALU = 256 * 4 * 16 * 2 * 2.4e9   # fp32 flop/s of the vector ALUs (FMA = 2), unpacked
 BIRUVIK_PATTERN = ("attention", "latent_attention", "hgrn2", "attention")
 BIRUVIK_RANK = 256    # latent size of the latent-attention layers
+# Lumepel: latent + rotated key part per size (key rows of 192 / 320 elements), query latent, experts
+LUMEPEL = {"s": dict(rank=128, rot=64, q_rank=384, experts=8, top=2, eff=1024),
+           "m": dict(rank=256, rot=64, q_rank=768, experts=16, top=2, eff=1408),
+           "l": dict(rank=256, rot=64, q_rank=1536, experts=32, top=4, eff=2048)}
+LUMEPEL_PATTERN = ("latent_attention", "latent_attention_2")
+BASELINE_OF = {"bidasun": "mistral", "biruvik": "mistral", "lumepel": "mixtral"}
 
 
 def _engine(kind: str, z: dict, max_len: int, pages: int, seqs: int):
     from nv_genai_amd.engine.llm_engine import EngineConfig, LLMEngine
-    from nv_genai_amd.models.config import LlamaConfig, bidasun_uniform, biruvik_layers
+    from nv_genai_amd.models.config import LlamaConfig, bidasun_uniform, biruvik_layers, lumepel_layers
 
-    if kind == "biruvik":
+    if kind == "lumepel":
+        u = z["lumepel"]
+        pat = [LUMEPEL_PATTERN[i % len(LUMEPEL_PATTERN)] for i in range(z["layers"])]
+        mcfg = lumepel_layers(pat, z["hidden"], z["heads"], z["d"], u["rot"], z["d"], u["rank"], u["q_rank"], 0,
+                              experts=u["experts"], top=u["top"], expert_ff=u["eff"], shared_ff=u["eff"],
+                              yarn=(8.0, 4096, 32.0, 1.0), vocab_size=VOCAB)
+    elif kind == "mixtral":
+        u = z["lumepel"]
+        mcfg = LlamaConfig(name="mixtral-eq", arch="mixtral", vocab_size=VOCAB, hidden=z["hidden"], layers=z["layers"],
+                           heads=z["heads"], kv_heads=z["kv"], head_dim=z["d"], ffn=u["eff"], num_experts=u["experts"],
+                           experts_per_tok=u["top"], max_position=max_len, rope_theta=1e6, eos_ids=(2,), bos_id=1)
+    elif kind == "biruvik":
         pat = [BIRUVIK_PATTERN[i % len(BIRUVIK_PATTERN)] for i in range(z["layers"])]
         mcfg = biruvik_layers(pat, z["hidden"], z["heads"], z["kv"], z["d"], z["d"], z["ffn"], window=z["window"],
                               kv_rank=BIRUVIK_RANK, vocab_size=VOCAB)
@@ -231,16 +249,126 @@ def biruvik_kernel_times(z: dict, iters: int = 20) -> dict:
     return out
 
 
+def lumepel_kernel_times(z: dict, iters: int = 20) -> dict:
+    """The Lumepel kernels alone on one layer's shapes beside the like kernels of the Llama layout:
+    latent attention (multi-query over the page of [latent | rotated key part] rows, values inside
+    the key rows) against causal softmax attention, the routed clamped-GLU experts against the
+    Mixtral experts, and the row kernels (latent norm + rotation + page write against rotation +
+    KV write; residual sum + norm; gated activation) against their counterparts, priced by the
+    bytes they must move."""
+    from nv_genai_amd import ops
+    from nv_genai_amd.ops import reference as ref
+
+    dev, bf = "cuda", torch.bfloat16
+    u = z["lumepel"]
+    H, G, D, R, RD = z["heads"], z["kv"], z["d"], u["rank"], u["rot"]
+    Wk = R + RD
+    nb, L = z["pf"]
+    nd, ctx = z["dec"]
+    pages_seq = -(-max(L, ctx) // 64)
+    nseq = max(nb, nd)
+    npg = nseq * pages_seq
+    bt = torch.arange(npg, dtype=torch.int32, device=dev).view(nseq, pages_seq)
+    page = (torch.randn(npg, 1, 64, Wk, device=dev) * 0.5).to(bf)
+    kl = (torch.randn(npg, G, 64, D, device=dev) * 0.5).to(bf)
+    vt = (torch.randn(npg, G, D, 64, device=dev) * 0.5).to(bf)
+    T = nb * L
+    cu = torch.arange(0, T + 1, L, dtype=torch.int32, device=dev)
+    cx = torch.full((nb,), L, dtype=torch.int32, device=dev)
+    ql = torch.randn(T, H * Wk, device=dev).to(bf)
+    q1 = torch.randn(T, H * D, device=dev).to(bf)
+    pairs = nb * (L * (L + 1) // 2) * H
+    sc = (D + RD) ** -0.5
+    out = {"mfma_attention": bool(ops.softmax_attention_mfma_ok(ql, Wk, R, H, 1))}
+    t_lat = _timed(lambda: ops.softmax_attention_prefill(ql, page, page, bt, cu, cx, L, H, 1, Wk, R, sc, v_in_k=True), iters)
+    t_soft = _timed(lambda: ops.prefill_attention_paged(q1, kl, vt, bt, cu, cx, H, G, D, L, D ** -0.5, window=0, impl=4),
+                    iters)
+    out["prefill"] = {"latent_ms": round(t_lat * 1e3, 3), "softmax_ms": round(t_soft * 1e3, 3),
+                      "latent_mfma_frac": round(2.0 * pairs * (Wk + R) / t_lat / PEAK_BF16, 4),
+                      "softmax_mfma_frac": round(4.0 * pairs * D / t_soft / PEAK_BF16, 4)}
+    seq = torch.arange(nd, dtype=torch.int32, device=dev)
+    pos = torch.full((nd,), ctx - 1, dtype=torch.int32, device=dev)
+    cxd = torch.full((nd,), ctx, dtype=torch.int32, device=dev)
+    ws = ops.DecodeWorkspace(nd, H, G, ctx, dev, None, D=D)
+    t_latd = _timed(lambda: ops.softmax_attention_rows(ql[:nd], page, page, bt, seq, pos, H, 1, Wk, R, sc, max_ctx=ctx,
+                                                       v_in_k=True), iters)
+    t_softd = _timed(lambda: ops.decode_attention(q1[:nd], kl, vt, bt, cxd, H, G, ctx, D ** -0.5, ws=ws, window=0), iters)
+    out["decode"] = {"latent_ms": round(t_latd * 1e3, 4), "softmax_ms": round(t_softd * 1e3, 4),
+                     "latent_hbm_frac": round(nd * ctx * Wk * 2.0 / t_latd / PEAK_HBM, 4),
+                     "softmax_hbm_frac": round(nd * G * ctx * 2 * D * 2.0 / t_softd / PEAK_HBM, 4)}
+    # ---- experts: T rows (prompts) and nd rows (single tokens)
+    Hd, E, k, F = z["hidden"], u["experts"], u["top"], u["eff"]
+    x = torch.randn(T, Hd, device=dev).to(bf)
+    router = (torch.randn(E, Hd, device=dev) * Hd ** -0.5)
+    w13 = (torch.randn(E, 2 * F, Hd, device=dev) * Hd ** -0.5).to(bf)
+    w2 = (torch.randn(E, Hd, F, device=dev) * F ** -0.5).to(bf)
+    rb = router.to(bf)
+
+    def lum(xx):
+        ids, wts = ops.moe_route_scores(ops.linear(xx.float(), router), k, "sigmoid", False)
+        return ops.moe_glu_experts(xx, ids, wts, w13, w2, 7.0, 1.702, True)
+
+    ex = {}
+    for name, rows in (("prefill", T), ("decode", nd)):
+        xx = x[:rows]
+        fl = 2.0 * rows * k * 3 * Hd * F
+        by = min(E, rows * k) * 3 * Hd * F * 2.0
+        t_l = _timed(lambda: lum(xx), iters)
+        t_m = _timed(lambda: ops.moe_ffn(xx, rb, w13, w2, k), iters)
+        ex[name] = {"lumepel_ms": round(t_l * 1e3, 3), "mixtral_ms": round(t_m * 1e3, 3),
+                    "lumepel_mfma_frac": round(fl / t_l / PEAK_BF16, 4), "mixtral_mfma_frac": round(fl / t_m / PEAK_BF16, 4),
+                    "lumepel_weight_hbm_frac": round(by / t_l / PEAK_HBM, 4),
+                    "mixtral_weight_hbm_frac": round(by / t_m / PEAK_HBM, 4)}
+    out["experts"] = ex
+    del x, w13, w2
+    # ---- row kernels (prompt rows): bytes that must move over the time, against 8 TB/s
+    nq = H * (D + RD)
+    proj = torch.randn(T, nq + Wk, device=dev).to(bf)
+    qf = torch.empty(T, H * Wk, device=dev, dtype=bf)
+    posr = torch.arange(L, dtype=torch.int32, device=dev).repeat(nb)
+    slots = torch.arange(T, dtype=torch.int32, device=dev)
+    freq, mag = ops.rotary_frequencies(RD, 1e4, (8.0, 4096, 32.0, 1.0))
+    freq = freq.to(dev)
+    cw = torch.ones(R, device=dev)
+    t_rc = _timed(lambda: ops.latent_rope_cache_(proj, posr, slots, page, freq, mag, True, RD, RD, 1e-5, kv=(nq, R, cw),
+                                                 q=(0, H, D), q_out=qf), iters)
+    by_rc = T * (2 * H * RD + 2 * Wk) * 2.0              # rotated parts read + written, latent row read + written
+    qkv = torch.randn(T, (H + 2 * G) * D, device=dev).to(bf)
+    cs = ref.rope_cos_sin(L, D, 1e6).to(dev)
+    t_rk = _timed(lambda: ops.rope_cache_(qkv, posr, cs, slots, kl, vt, H, G, D), iters)
+    by_rk = T * (2 * (H + G) * D + 2 * G * D) * 2.0      # q, k read + written, k and v pages written, v read
+    xs = torch.randn(T, Hd, device=dev)
+    y = torch.randn(T, Hd, device=dev).to(bf)
+    wn = torch.ones(Hd, device=dev)
+    t_rn = _timed(lambda: ops.residual_add_rmsnorm_(xs, y, wn, 1e-5, bf), iters)
+    xb = xs.to(bf)
+    wb = wn.to(bf)
+    t_an = _timed(lambda: ops.add_rmsnorm(xb, y, wb, 1e-5), iters)
+    Fd = 4 * Hd
+    gu = torch.randn(T, 2 * Fd, device=dev).to(bf)
+    t_cg = _timed(lambda: ops.clamped_glu(gu, Fd, 7.0), iters)
+    t_sm = _timed(lambda: ops.silu_mul(gu), iters)
+    out["rows"] = {
+        "latent_rope_cache_ms": round(t_rc * 1e3, 3), "latent_rope_cache_hbm_frac": round(by_rc / t_rc / PEAK_HBM, 4),
+        "rope_cache_ms": round(t_rk * 1e3, 3), "rope_cache_hbm_frac": round(by_rk / t_rk / PEAK_HBM, 4),
+        "residual_add_rmsnorm_ms": round(t_rn * 1e3, 3),
+        "residual_add_rmsnorm_hbm_frac": round(T * Hd * 12.0 / t_rn / PEAK_HBM, 4),     # fp32 in + out, bf16 in + out
+        "add_rmsnorm_ms": round(t_an * 1e3, 3), "add_rmsnorm_hbm_frac": round(T * Hd * 8.0 / t_an / PEAK_HBM, 4),
+        "clamped_glu_ms": round(t_cg * 1e3, 3), "clamped_glu_hbm_frac": round(T * Fd * 6.0 / t_cg / PEAK_HBM, 4),
+        "silu_mul_ms": round(t_sm * 1e3, 3), "silu_mul_hbm_frac": round(T * Fd * 6.0 / t_sm / PEAK_HBM, 4)}
+    return out
+
+
 def run(args) -> None:
     names = [s for s in (args.design_sizes or "s,m,l").split(",") if s]
     models = [m for m in (getattr(args, "design_models", None) or "bidasun").split(",") if m]
-    if any(m not in ("bidasun", "biruvik") for m in models):
-        raise SystemExit(f"--design-models: unknown design in {models} (bidasun, biruvik)")
+    if any(m not in BASELINE_OF for m in models):
+        raise SystemExit(f"--design-models: unknown design in {models} ({', '.join(BASELINE_OF)})")
     res = {}
     for n in names:
-        z = SIZES[n]
+        z = dict(SIZES[n], lumepel=LUMEPEL[n])
         res[n] = {"shape": {k: v for k, v in z.items()}}
-        for kind in models + ["mistral"]:
+        for kind in models + sorted({BASELINE_OF[m] for m in models}):
             res[n][kind] = engine_rates(kind, z, max(1, args.steps), max(1, args.warmup))
             torch.cuda.empty_cache()
         if "bidasun" in models:
@@ -248,6 +376,9 @@ def run(args) -> None:
             torch.cuda.empty_cache()
         if "biruvik" in models:
             res[n]["biruvik_kernels"] = biruvik_kernel_times(z)
+            torch.cuda.empty_cache()
+        if "lumepel" in models:
+            res[n]["lumepel_kernels"] = lumepel_kernel_times(z)
             torch.cuda.empty_cache()
         print(f"[designs] {n}: {json.dumps(res[n])}", flush=True)
     line = {"metric": "design_compare", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

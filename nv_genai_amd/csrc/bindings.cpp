@@ -1516,7 +1516,8 @@ const FormSpec kForms[KF_COUNT] = {
     {"decode_dma", "NGA_DECODE_DMA", 2}, {"decode_nt", "NGA_DECODE_NT", 2},
     {"search_dma", "NGA_SEARCH_DMA", 1}, {"prefill_v1", "NGA_PREFILL_V1", 0},
     {"prefill_ks", "NGA_PREFILL_KS", 0}, {"rope_vnt", "NGA_ROPE_VNT", 2},
-    {"decode_dma_aux", "NGA_DECODE_DMA_AUX", 2}, {"sig_decode_waves", "NGA_SIG_DECODE_WAVES", 8192}};
+    {"decode_dma_aux", "NGA_DECODE_DMA_AUX", 2}, {"sig_decode_waves", "NGA_SIG_DECODE_WAVES", 8192},
+    {"sm_share_heads", "NGA_SM_SHARE_HEADS", 1}};
 std::atomic<int>* forms() {
   static std::atomic<int> v[KF_COUNT];
   static const bool init = [] {

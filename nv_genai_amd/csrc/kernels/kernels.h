@@ -18,6 +18,7 @@ enum KernelForm {
   KF_ROPE_VNT,         // NGA_ROPE_VNT: non-temporal 2-byte V^T page stores in the RoPE / KV-write kernels: 1 all, 2 tokens with no same-page neighbour
   KF_DECODE_DMA_AUX,   // NGA_DECODE_DMA_AUX: cache policy of the LDS-DMA decode kernel's KV loads: 2 nt (default), 0 default policy
   KF_SIG_DECODE_WAVES, // NGA_SIG_DECODE_WAVES: waves the single-token sigmoid attention kernel aims to launch (sets its parts)
+  KF_SM_SHARE_HEADS,   // NGA_SM_SHARE_HEADS: prompt softmax attention over a latent page (keys 96 / 192 / 320 wide): 0 one head per wave, 1 two heads per wave over one K tile (default; 96- and 192-wide keys)
   KF_COUNT
 };
 int kernel_form(KernelForm f);

@@ -1,4 +1,4 @@
-// Projection-side kernel of latent attention with a rotated key part (one workgroup per token):
+// Projection-side kernel of latent attention with a rotated key part (one wave per token):
 //
 //   * optional RMS norm, in place, of a column range (a query latent in front of its
 //     up-projection);
@@ -19,7 +19,6 @@ namespace nga {
 
 namespace {
 
-constexpr int BS = 64;          // tokens per page
 constexpr int MAX_PAIRS = 256;  // rot_dims <= 512
 
 template <typename T> __device__ __forceinline__ float ldf(const T* p);
@@ -51,15 +50,19 @@ __device__ __forceinline__ float rotated(const T* src, int e, int n, bool interl
   return first ? a * cs[pair] - b * sn[pair] : a * cs[pair] + b * sn[pair];
 }
 
+// One wave per token, four tokens per workgroup: the norm statistics are wave reductions and the
+// cos / sin of the token live in the wave's own LDS rows, so no workgroup barrier is needed.
 template <typename T>
-__global__ void __launch_bounds__(256) latent_rope_cache_kernel(const LatentRopeParams P) {
-  __shared__ float cs[MAX_PAIRS], sn[MAX_PAIRS];
-  __shared__ float red[4];
-  const int64_t row = blockIdx.x;
-  const int tid = threadIdx.x;
+__global__ void __launch_bounds__(256) latent_rope_cache_kernel(const LatentRopeParams P, int64_t T_rows) {
+  __shared__ float cs_all[4][MAX_PAIRS], sn_all[4][MAX_PAIRS];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+  if (row >= T_rows) return;
+  float* cs = cs_all[wave];
+  float* sn = sn_all[wave];
   T* pr = (T*)P.proj + row * P.stride;
   const int p = P.pos[row] < 0 ? 0 : P.pos[row];
-  for (int i = tid; i < P.rot_dims / 2; i += blockDim.x) {
+  for (int i = lane; i < P.rot_dims / 2; i += 64) {
     const double turns = (double)p * P.freq[i] * 0.15915494309189535;   // angle / 2 pi
     const float a = (float)((turns - floor(turns)) * 6.283185307179586);
     float s, c;
@@ -69,39 +72,60 @@ __global__ void __launch_bounds__(256) latent_rope_cache_kernel(const LatentRope
   }
   if (P.n_off >= 0) {
     float ss = 0.f;
-    for (int c = tid; c < P.n_n; c += blockDim.x) {
+    for (int c = lane; c < P.n_n; c += 64) {
       const float v = ldf(pr + P.n_off + c);
       ss += v * v;
     }
-    ss = block_sum(ss, red);
+    ss = wave_sum(ss);
     const float r = 1.0f / sqrtf(ss / (float)P.n_n + P.eps);
-    for (int c = tid; c < P.n_n; c += blockDim.x) stf(pr + P.n_off + c, ldf(pr + P.n_off + c) * r * P.n_w[c]);
+    for (int c = lane; c < P.n_n; c += 64) stf(pr + P.n_off + c, ldf(pr + P.n_off + c) * r * P.n_w[c]);
   }
-  __syncthreads();
+  __builtin_amdgcn_wave_barrier();   // the wave's cos / sin rows are written (LDS ops of a wave complete in order)
   if (P.kv_off >= 0) {
-    float ss = 0.f;
-    for (int c = tid; c < P.r; c += blockDim.x) {
-      const float v = ldf(pr + P.kv_off + c);
-      ss += v * v;
-    }
-    ss = block_sum(ss, red);
     const int slot = P.slots[row];
     if (slot >= 0) {
+      float ss = 0.f;
+      for (int c = lane; c < P.r; c += 64) {
+        const float v = ldf(pr + P.kv_off + c);
+        ss += v * v;
+      }
+      ss = wave_sum(ss);
       const float r = 1.0f / sqrtf(ss / (float)P.r + P.eps);
-      T* dst = (T*)P.page + ((int64_t)(slot / BS) * BS + slot % BS) * (P.r + P.rot_dim);
-      for (int c = tid; c < P.r; c += blockDim.x) stf(dst + c, ldf(pr + P.kv_off + c) * r * P.kv_w[c]);
+      T* dst = (T*)P.page + (int64_t)slot * (P.r + P.rot_dim);   // page rows are contiguous: slot = page * 64 + offset
+      for (int c = lane; c < P.r; c += 64) stf(dst + c, ldf(pr + P.kv_off + c) * r * P.kv_w[c]);
       const T* kr = pr + P.kv_off + P.r;
-      for (int e = tid; e < P.rot_dim; e += blockDim.x)
+      for (int e = lane; e < P.rot_dim; e += 64)
         stf(dst + P.r + e, rotated(kr, e, P.rot_dims, P.interleaved != 0, cs, sn));
     }
   }
   if (P.q_off >= 0) {
+    // element e of every head's rotated part: the pair, its partner and cos / sin are the lane's
+    // own for all heads
     const int qd = P.dim + P.rot_dim;
-    T* qo = (T*)P.q_out + row * P.q_out_stride;
-    for (int i = tid; i < P.heads * P.rot_dim; i += blockDim.x) {
-      const int h = i / P.rot_dim, e = i - h * P.rot_dim;
-      stf(qo + (int64_t)h * P.q_w + (P.q_w - P.rot_dim) + e,
-          rotated(pr + P.q_off + (int64_t)h * qd + P.dim, e, P.rot_dims, P.interleaved != 0, cs, sn));
+    T* qo = (T*)P.q_out + row * P.q_out_stride + (P.q_w - P.rot_dim);
+    const T* qi = pr + P.q_off + P.dim;
+    for (int e = lane; e < P.rot_dim; e += 64) {
+      if (e >= P.rot_dims) {
+        for (int h = 0; h < P.heads; ++h) stf(qo + (int64_t)h * P.q_w + e, ldf(qi + (int64_t)h * qd + e));
+        continue;
+      }
+      int pair, other;
+      bool first;
+      if (P.interleaved) {
+        pair = e >> 1;
+        first = (e & 1) == 0;
+        other = e ^ 1;
+      } else {
+        const int half = P.rot_dims >> 1;
+        first = e < half;
+        pair = first ? e : e - half;
+        other = first ? e + half : e - half;
+      }
+      const float c = cs[pair], s = first ? -sn[pair] : sn[pair];
+      for (int h = 0; h < P.heads; ++h) {
+        const T* src = qi + (int64_t)h * qd;
+        stf(qo + (int64_t)h * P.q_w + e, ldf(src + e) * c + ldf(src + other) * s);
+      }
     }
   }
 }
@@ -111,10 +135,11 @@ __global__ void __launch_bounds__(256) latent_rope_cache_kernel(const LatentRope
 void launch_latent_rope_cache(const LatentRopeParams& p, int64_t T, bool f32, hipStream_t stream) {
   if (T == 0) return;
   if (p.rot_dims / 2 > MAX_PAIRS) abort();   // the binding checks rot_dims <= 512
+  const dim3 grid((unsigned)((T + 3) / 4));
   if (f32)
-    latent_rope_cache_kernel<float><<<dim3((unsigned)T), 256, 0, stream>>>(p);
+    latent_rope_cache_kernel<float><<<grid, 256, 0, stream>>>(p, T);
   else
-    latent_rope_cache_kernel<uint16_t><<<dim3((unsigned)T), 256, 0, stream>>>(p);
+    latent_rope_cache_kernel<uint16_t><<<grid, 256, 0, stream>>>(p, T);
 }
 
 }  // namespace nga

@@ -329,9 +329,10 @@ __global__ void __launch_bounds__(256) moe_gemm_kernel(MoeGemmParams P) {
 }
 
 // ------------------------------------------------------------------ combine
-// out[t, :] = sum_j y[inv[t*k + j], :] (fp32), 8 features per thread
+// out[t, :] = sum_j y[inv[t*k + j], :] (+ add[t, :]) (fp32), 8 features per thread
 __global__ void moe_combine_kernel(const uint16_t* __restrict__ y, const int32_t* __restrict__ inv,
-                                   int T, int k, int H, uint16_t* __restrict__ out) {
+                                   int T, int k, int H, uint16_t* __restrict__ out,
+                                   const uint16_t* __restrict__ add = nullptr, int64_t add_stride = 0) {
   const int64_t vec = H / 8;
   const int64_t total = (int64_t)T * vec;
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
@@ -339,6 +340,11 @@ __global__ void moe_combine_kernel(const uint16_t* __restrict__ y, const int32_t
     const int64_t t = i / vec;
     const int c = (int)(i - t * vec) * 8;
     float a[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (add) {
+      const u16x8 v = load8(add + t * add_stride + c);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) a[q] = bf2f(v[q]);
+    }
     for (int j = 0; j < k; ++j) {
       const int p = inv[t * k + j];
       if (p < 0) continue;
@@ -568,6 +574,13 @@ void launch_moe_gemm_rows(const MoeRowsParams& p, int mode, bool f32, hipStream_
 void launch_moe_combine_rows(const void* y, const int32_t* inv, int T, int k, int H, const void* add,
                              int64_t add_stride, void* out, bool f32, hipStream_t stream) {
   if (T == 0) return;
+  if (!f32 && H % 8 == 0 && (add == nullptr || (add_stride % 8 == 0 && ((uintptr_t)add % 16) == 0))) {
+    int64_t g = ((int64_t)T * H / 8 + 255) / 256;
+    if (g > 4096) g = 4096;
+    moe_combine_kernel<<<(unsigned)g, 256, 0, stream>>>((const uint16_t*)y, inv, T, k, H, (uint16_t*)out,
+                                                        (const uint16_t*)add, add_stride);
+    return;
+  }
   if (f32)
     moe_combine_rows_kernel<float><<<T, 256, 0, stream>>>((const float*)y, inv, k, H, (const float*)add, add_stride,
                                                          (float*)out);

@@ -227,6 +227,28 @@ __global__ void __launch_bounds__(256) clamped_glu_kernel(T* __restrict__ out, c
   }
 }
 
+// bf16 rows with F % 8 == 0 and 16-byte aligned rows: 8 gates and 8 ups per thread
+__global__ void __launch_bounds__(256) clamped_glu_bf16x8_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ in,
+                                                                 int64_t in_stride, int64_t T_rows, int F8, float limit,
+                                                                 float alpha, int gate_col) {
+  const int64_t total = T_rows * F8;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = i / F8;
+    const int c = (int)(i - t * F8) * 8;
+    const uint16_t* r = in + t * in_stride;
+    const u16x8 g8 = load8(r + c), u8 = load8(r + 8 * F8 + c);
+    const float rg = gate_col >= 0 ? 1.0f / (1.0f + expf(-bf2f(r[gate_col]))) : 1.0f;
+    u16x8 o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float g = fminf(bf2f(g8[j]), limit);
+      const float u = fminf(fmaxf(bf2f(u8[j]), -limit), limit);
+      o[j] = f2bf(g / (1.0f + expf(-alpha * g)) * (u + 1.0f) * rg);
+    }
+    store8(out + t * 8 * F8 + c, o);
+  }
+}
+
 __global__ void __launch_bounds__(256) softcap_kernel(float* __restrict__ z, int64_t n, float cap, float inv) {
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
     z[i] = cap * tanhf(z[i] * inv);
@@ -364,6 +386,13 @@ void launch_residual_add_rmsnorm(float* x, const void* y, int64_t y_stride, cons
 void launch_clamped_glu(void* out, const void* in, int64_t in_stride, int64_t T, int F, float limit, float alpha,
                         int gate_col, bool f32, hipStream_t stream) {
   if (T == 0 || F == 0) return;
+  if (!f32 && F % 8 == 0 && in_stride % 8 == 0 && ((uintptr_t)in % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+    int64_t g8 = (T * (F / 8) + 255) / 256;
+    if (g8 > 16384) g8 = 16384;
+    clamped_glu_bf16x8_kernel<<<dim3((unsigned)g8), 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)in, in_stride, T,
+                                                                      F / 8, limit, alpha, gate_col);
+    return;
+  }
   int64_t g = (T * F + 255) / 256;
   if (g > 8192) g = 8192;
   if (f32)

@@ -234,9 +234,15 @@ struct SmMfmaParams {
 // WPE: waves per SIMD the register allocation aims at. Large tiles (maps x DK + DV >= 192) are
 // compiled for two: with the whole register file the scheduler keeps a tile's LDS reads in flight
 // ahead of the MFMAs instead of reading fragment by fragment (2x faster at 128-wide heads, measured).
-template <int DK, int DV, int MAPS, int WPE>
+// SHARE (MAPS = 2): the wave's two score maps are two *heads* (2 hq, 2 hq + 1) of one KV head that
+// read the same K tile - every K fragment is read from LDS once for both heads' MFMAs, as the V^T
+// fragments are - and their outputs are written separately. With many heads over one page
+// (multi-query attention over a latent) this halves the staging and the LDS reads per flop.
+template <int DK, int DV, int MAPS, int WPE, bool SHARE = false>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 softmax_attention_mfma_kernel(const SmMfmaParams P) {
+  static_assert(!SHARE || MAPS == 2, "two heads per wave");
+  constexpr int KM = SHARE ? 1 : MAPS;     // K tiles staged per page
   constexpr int KT = 64;
   constexpr int NCH_K = DK / 8;
   constexpr int DS = DK / 32;
@@ -248,14 +254,14 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
   constexpr int P2 = NCH_K & -NCH_K;
   constexpr int SWS = P2 >= 16 ? 0 : P2 == 8 ? 1 : 2;
   extern __shared__ __attribute__((aligned(16))) uint16_t sm_lds[];
-  uint16_t* k_s = sm_lds;                       // [MAPS][KT * DK]
-  uint16_t* v_s = sm_lds + MAPS * KT * DK;      // [DV * KT]
+  uint16_t* k_s = sm_lds;                       // [KM][KT * DK]
+  uint16_t* v_s = sm_lds + KM * KT * DK;        // [DV * KT]
   // the last row blocks of a sequence see the most pages: they are launched first
   const int tile = gridDim.x - 1 - blockIdx.x, hq = blockIdx.y, b = blockIdx.z;
   const int q0 = P.cu_q[b], qlen = P.cu_q[b + 1] - q0;
   if (tile * 64 >= qlen) return;
   const int ctx = P.ctx_lens[b];
-  const int g = hq / (P.H / P.G);
+  const int g = (SHARE ? 2 * hq : hq) / (P.H / P.G);
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15, h = lane >> 4;
@@ -294,14 +300,14 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
 
   // Registers for one page in flight: with few enough of them the next page is requested before
   // the current one is processed, so its latency hides behind the MFMA work.
-  constexpr bool PREFETCH = (MAPS * PER_K + 4 * VBLK) * 4 <= 48;
-  u16x8 kreg[MAPS][PER_K], vreg[VBLK][4];
+  constexpr bool PREFETCH = (KM * PER_K + 4 * VBLK) * 4 <= 48;
+  u16x8 kreg[KM][PER_K], vreg[VBLK][4];
   auto fetch = [&](int t) {
     const int64_t blk = P.block_tables[(int64_t)b * P.max_blocks + t];
-    const uint16_t* kp = P.kc + (blk * P.G + g) * (int64_t)(MAPS * KT * DK);
+    const uint16_t* kp = P.kc + (blk * P.G + g) * (int64_t)(KM * KT * DK);
     const uint16_t* vp = P.vc + (blk * P.G + g) * (int64_t)KT * P.v_row;
 #pragma unroll
-    for (int m = 0; m < MAPS; ++m)
+    for (int m = 0; m < KM; ++m)
 #pragma unroll
       for (int i = 0; i < PER_K; ++i) kreg[m][i] = load8(kp + m * KT * DK + (int64_t)(tid + 256 * i) * 8);
 #pragma unroll
@@ -317,7 +323,7 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
   for (int t = t_first; t <= t_last; ++t) {
     __syncthreads();   // the previous page's reads are done
 #pragma unroll
-    for (int m = 0; m < MAPS; ++m)
+    for (int m = 0; m < KM; ++m)
 #pragma unroll
       for (int i = 0; i < PER_K; ++i) {
         const int c = tid + 256 * i;
@@ -349,19 +355,40 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
     const float fd = (float)(qpos - kbase - 8 * h);
     const bool need_mask = kbase + KT - 1 > wq_lo || (W > 0 && wq_hi - kbase >= W);
     bf16x8 pf[MAPS][2];
+    f32x4 sboth[SHARE ? MAPS : 1][4];
+    if constexpr (SHARE) {   // both heads' scores from one read of every K fragment
+#pragma unroll
+      for (int tau = 0; tau < 4; ++tau) {
+        const int row = 32 * (tau >> 1) + 8 * (col >> 2) + 4 * (tau & 1) + (col & 3);
+        const int sw = sm_row_swz(row) >> SWS;
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m) sboth[m][tau] = (f32x4)(0.f);
+#pragma unroll
+        for (int s2 = 0; s2 < DS; ++s2) {
+          const int ch = 4 * s2 + h;
+          const bf16x8 a = as_bf16x8(*reinterpret_cast<const u16x8*>(&k_s[row * DK + ((ch ^ sw) * 8)]));
+#pragma unroll
+          for (int m = 0; m < MAPS; ++m) sboth[m][tau] = mfma16(a, qf[m][s2], sboth[m][tau]);
+        }
+      }
+    }
 #pragma unroll
     for (int m = 0; m < MAPS; ++m) {
       f32x4 sacc[4];
 #pragma unroll
       for (int tau = 0; tau < 4; ++tau) {
-        const int row = 32 * (tau >> 1) + 8 * (col >> 2) + 4 * (tau & 1) + (col & 3);
-        const int sw = sm_row_swz(row) >> SWS;
-        sacc[tau] = (f32x4)(0.f);
+        if constexpr (SHARE) {
+          sacc[tau] = sboth[m][tau];
+        } else {
+          const int row = 32 * (tau >> 1) + 8 * (col >> 2) + 4 * (tau & 1) + (col & 3);
+          const int sw = sm_row_swz(row) >> SWS;
+          sacc[tau] = (f32x4)(0.f);
 #pragma unroll
-        for (int s2 = 0; s2 < DS; ++s2) {
-          const int ch = 4 * s2 + h;
-          const bf16x8 a = as_bf16x8(*reinterpret_cast<const u16x8*>(&k_s[m * KT * DK + row * DK + ((ch ^ sw) * 8)]));
-          sacc[tau] = mfma16(a, qf[m][s2], sacc[tau]);
+          for (int s2 = 0; s2 < DS; ++s2) {
+            const int ch = 4 * s2 + h;
+            const bf16x8 a = as_bf16x8(*reinterpret_cast<const u16x8*>(&k_s[m * KT * DK + row * DK + ((ch ^ sw) * 8)]));
+            sacc[tau] = mfma16(a, qf[m][s2], sacc[tau]);
+          }
         }
       }
       float mx = -INFINITY;
@@ -418,6 +445,39 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
   float inv[MAPS];
 #pragma unroll
   for (int m = 0; m < MAPS; ++m) inv[m] = 1.0f / lrun[m];
+  if constexpr (SHARE) {   // two heads: each normalised, scaled, gated and written on its own
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+      float s2 = 0.f;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          const float v = o[m][dt][rr] * inv[m];
+          o[m][dt][rr] = v;
+          s2 += v * v;
+        }
+      float rs = 1.0f;
+      if (P.unit_eps >= 0.f) {
+        s2 += __shfl_xor(s2, 16, 64);
+        s2 += __shfl_xor(s2, 32, 64);
+        rs = P.out_scale / sqrtf(s2 / (float)DV + P.unit_eps);
+      }
+      if (row_ok) {
+        const int head = 2 * hq + m;
+        if (P.gate) rs *= sigmoidf_(bf2f(P.gate[(int64_t)(q0 + r) * P.g_stride + head]));
+        uint16_t* op = P.out + (int64_t)(q0 + r) * P.H * DV + (int64_t)head * DV;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          u16x4 ov;
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) ov[rr] = f2bf(o[m][dt][rr] * rs);
+          *reinterpret_cast<u16x4*>(op + 16 * dt + 4 * h) = ov;
+        }
+      }
+    }
+    return;
+  }
   float ss = 0.f;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
@@ -475,10 +535,27 @@ bool launch_sm_mfma_dv(const SmMfmaParams& P, int dv, dim3 grid, hipStream_t str
   }
 }
 
-// key sizes of a latent plus a rotated part (one map): one value size each
+// two heads of one KV head per wave over a shared K tile (one map per head)
 template <int DK, int DV>
+void launch_sm_mfma_shared(const SmMfmaParams& P, dim3 grid, hipStream_t stream) {
+  constexpr size_t smem = (size_t)(64 * DK + DV * 64) * sizeof(uint16_t);
+  static_assert(smem <= 65536, "dynamic LDS without the attribute");
+  grid.y = (unsigned)(P.H / 2);
+  softmax_attention_mfma_kernel<DK, DV, 2, 2, true><<<grid, 256, smem, stream>>>(P);
+}
+
+// key sizes of a latent plus a rotated part (one map): one value size each. SHARED: an even number
+// of heads per KV head runs two heads per wave (both heads' accumulators fit two waves per SIMD;
+// at 320-wide keys they do not, and one wave per SIMD measured twice as slow as one head per wave).
+template <int DK, int DV, bool SHARED>
 bool launch_sm_mfma_pair(const SmMfmaParams& P, int dv, dim3 grid, hipStream_t stream) {
   if (dv != DV) return false;
+  if constexpr (SHARED) {
+    if (kernel_form(KF_SM_SHARE_HEADS) != 0 && (P.H / P.G) % 2 == 0) {
+      launch_sm_mfma_shared<DK, DV>(P, grid, stream);
+      return true;
+    }
+  }
   launch_sm_mfma_one<DK, DV, 1>(P, grid, stream);
   return true;
 }
@@ -486,9 +563,9 @@ bool launch_sm_mfma_pair(const SmMfmaParams& P, int dv, dim3 grid, hipStream_t s
 template <int MAPS>
 bool launch_sm_mfma_dk(const SmMfmaParams& P, int dk, int dv, dim3 grid, hipStream_t stream) {
   if (MAPS == 1) {
-    if (dk == 96) return launch_sm_mfma_pair<96, 64>(P, dv, grid, stream);
-    if (dk == 192) return launch_sm_mfma_pair<192, 128>(P, dv, grid, stream);
-    if (dk == 320) return launch_sm_mfma_pair<320, 256>(P, dv, grid, stream);
+    if (dk == 96) return launch_sm_mfma_pair<96, 64, true>(P, dv, grid, stream);
+    if (dk == 192) return launch_sm_mfma_pair<192, 128, true>(P, dv, grid, stream);
+    if (dk == 320) return launch_sm_mfma_pair<320, 256, false>(P, dv, grid, stream);
   }
   switch (dk) {
     case 32: return launch_sm_mfma_dv<32, MAPS>(P, dv, grid, stream);

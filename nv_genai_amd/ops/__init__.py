@@ -776,7 +776,7 @@ class DecodeWorkspace:
 
 
 KERNEL_FORMS = ("decode_dma", "decode_nt", "search_dma", "prefill_v1", "prefill_ks", "rope_vnt",
-                "decode_dma_aux", "sig_decode_waves")
+                "decode_dma_aux", "sig_decode_waves", "sm_share_heads")
 
 
 def kernel_form(name: str) -> int:
