@@ -181,12 +181,12 @@ void moe_align(Tensor ids, Tensor w, int64_t T, int64_t k, int64_t e0, int64_t E
   CHECK_DEV(sorted_w); CHECK_DT(sorted_w, at::kFloat);
   CHECK_DEV(inv); CHECK_DT(inv, at::kInt);
   CHECK_DEV(tiles); CHECK_DT(tiles, at::kInt);
-  TORCH_CHECK(E >= 1 && E <= 256 && (bm == 64 || bm == 128) && e0 >= 0);
+  TORCH_CHECK(E >= 1 && E <= 512 && (bm == 64 || bm == 128) && e0 >= 0);
   TORCH_CHECK(ids.numel() >= M && w.numel() >= M && sorted_tok.numel() >= M &&
               sorted_w.numel() >= M && inv.numel() >= M && tiles.numel() >= 3 * mt_cap);
   // every expert's rows fit the table: sum_e ceil(cnt_e / bm) <= M / bm + E
   TORCH_CHECK(mt_cap >= (M + bm - 1) / bm + E, "moe_align: M-tile table too small");
-  TORCH_CHECK(k >= 1 && k <= 8);
+  TORCH_CHECK(k >= 1 && k <= 16);
   nga::launch_moe_align(ids.data_ptr<int32_t>(), w.data_ptr<float>(), (int)M, (int)k, (int)e0, (int)E,
                         (int)bm, sorted_tok.data_ptr<int32_t>(), sorted_w.data_ptr<float>(),
                         inv.data_ptr<int32_t>(), tiles.data_ptr<int32_t>(), (int)mt_cap,
@@ -247,7 +247,7 @@ void moe_route_scores(Tensor logits, int64_t k, int64_t score, bool renorm, Tens
   CHECK_DEV(logits); CHECK_DT(logits, at::kFloat);
   TORCH_CHECK(logits.dim() == 2 && logits.stride(1) == 1, "moe_route_scores: logits must be [T, E]");
   const int64_t T = logits.size(0), E = logits.size(1);
-  TORCH_CHECK(E >= 1 && E <= 256 && k >= 1 && k <= 8 && k <= E, "moe_route_scores: 1 <= k <= min(8, E), E <= 256");
+  TORCH_CHECK(E >= 1 && E <= 512 && k >= 1 && k <= 16 && k <= E, "moe_route_scores: 1 <= k <= min(16, E), E <= 512");
   TORCH_CHECK(score == 0 || score == 1);
   CHECK_DEV(ids); CHECK_DT(ids, at::kInt); CHECK_DEV(w); CHECK_DT(w, at::kFloat);
   TORCH_CHECK(ids.is_contiguous() && w.is_contiguous() && ids.numel() >= T * k && w.numel() >= T * k);
@@ -1400,8 +1400,8 @@ SoftmaxArgs check_softmax_args(const Tensor& out, const Tensor& q, const c10::op
   TORCH_CHECK(maps == 1 || maps == 2, "softmax_attention: one or two maps per head");
   TORCH_CHECK(q.dim() == 2 && q.stride(1) == 1 && q.size(1) == H * maps * dk, "q must be [T, H * maps * dk] rows");
   TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == H * dv);
-  TORCH_CHECK(H > 0 && G > 0 && H % G == 0 && dk > 0 && dk <= 2048 && dv > 0 && dv <= 512 && window >= 0,
-              "softmax_attention: dk <= 2048, dv <= 512");
+  TORCH_CHECK(H > 0 && G > 0 && H % G == 0 && dk > 0 && dk <= 2048 && dv > 0 && dv <= 1024 && window >= 0,
+              "softmax_attention: dk <= 2048, dv <= 1024");
   check_row_pages(q, kc, G * maps, dk, "softmax_attention (k)");
   if (v_in_k) {
     TORCH_CHECK(maps == 1 && dv <= dk && vc.data_ptr() == kc.data_ptr(),

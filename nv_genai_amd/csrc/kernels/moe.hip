@@ -38,7 +38,7 @@ namespace nga {
 
 namespace {
 constexpr int BK = 64;   // K per stage (one 128-B row of bf16)
-constexpr int MAX_E = 256;
+constexpr int MAX_E = 512;
 
 __device__ __forceinline__ int swz(int row, int ch) {  // 16-B chunk position in a 128-B LDS row
   return row * BK + ((ch ^ ((row >> 1) & 7)) << 3);
@@ -369,8 +369,8 @@ __global__ void moe_route_scores_kernel(const float* __restrict__ logits, int64_
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
   const float* lp = logits + (int64_t)t * ld;
-  float top[8];
-  int sel[8];
+  float top[16];
+  int sel[16];
   for (int j = 0; j < k; ++j) {
     float best = -INFINITY;
     int bi = -1;

@@ -143,8 +143,10 @@ __global__ void __launch_bounds__(64) softmax_attention_kernel(
   const int g = h / (H / G);
   const int32_t* bt = block_tables + (int64_t)seq * max_blocks;
   for (int d = lane; d < maps * dk; d += 64) qs[d] = ldf(q + row * q_stride + (int64_t)h * maps * dk + d);
-  constexpr int MAXV = 8;   // dv <= 512
-  float res[MAXV] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, acc[MAXV];
+  constexpr int MAXV = 16;   // dv <= 1024
+  float res[MAXV], acc[MAXV];
+#pragma unroll
+  for (int u = 0; u < MAXV; ++u) res[u] = 0.f;
   const int lo = window > 0 && i - window + 1 > 0 ? i - window + 1 : 0;
   const int p_lo = lo / BS, p_hi = i / BS;
   const bool vec = (dk % (16 / (int)sizeof(T))) == 0;

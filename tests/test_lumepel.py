@@ -151,9 +151,10 @@ def test_stream_ops_glu_softcap(device, dtype):
     close(h, O.rmsnorm(xs, w.double(), 1e-5), dtype, "norm of the sum")
     assert ops.residual_add_rmsnorm_(x, y.to(device), None, 1e-5, tdt) is None
     close(x, xs + y.double(), "float32", "sum only")
-    # clamped GLU: values on both sides of the limits, a gate column behind padding
-    gu = (3.0 * torch.randn(T, 2 * F + 3, generator=g)).to(tdt)
-    for lim in (0.5, 7.0):
+    # clamped GLU: values on both sides of the limits, a gate column behind padding; widths the
+    # 8-wide form takes and widths it does not
+    for F, pad, lim in ((23, 3, 0.5), (23, 3, 7.0), (24, 8, 0.5), (24, 8, 7.0)):
+        gu = (3.0 * torch.randn(T, 2 * F + pad, generator=g)).to(tdt)
         a = ops.clamped_glu(gu.to(device), F, lim, GLU_ALPHA)
         gg, uu = gu[:, :F].double().clamp(max=lim), gu[:, F:2 * F].double().clamp(-lim, lim)
         want = gg * torch.sigmoid(1.702 * gg) * (uu + 1.0)
@@ -224,7 +225,8 @@ def o_attention_in_keys(q, rows, dv, scale, pos):
     return out.reshape(T, H * dv)
 
 
-@pytest.mark.parametrize("shape", [(3, 26, 20), (18, 96, 64), (4, 192, 128), (2, 320, 256), (1, 13, 13)])
+@pytest.mark.parametrize("shape", [(3, 26, 20), (18, 96, 64), (4, 192, 128), (2, 320, 256), (1, 13, 13), (2, 64, 32),
+                                   (3, 128, 64), (2, 256, 128), (1, 600, 530)])
 @pytest.mark.parametrize("device,dtype", DTYPES)
 def test_one_key_stands_out_and_random(device, dtype, shape):
     """Values read out of the key rows. One key row is made to match a scaled query, far back,
