@@ -51,7 +51,7 @@ class LumepelModel:
     stateful = True                # steps carry the engine's row maps (block-table row of every token)
     uses_decode_workspace = False
     supports_step_graphs = False   # prefill / mixed steps run eagerly (decode steps are graphs)
-    supports_prefix_cache = False
+    supports_prefix_cache = True   # a page holds everything a token leaves behind
 
     def __init__(self, cfg: LumepelConfig, device="cuda", dtype=torch.bfloat16,
                  pctx: Optional[ParallelContext] = None, seed: int = 0,

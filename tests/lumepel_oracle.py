@@ -117,13 +117,15 @@ def route(h, w_router, top):
 def moe_ff(h, w, p, mlp):
     """Sum over a token's experts of expert(weight * h), plus the shared expert times a sigmoid
     gate of one number per token."""
-    idx, val = route(h, w[p + "mlp.router"], int(mlp["router"]["top"]))
+    top = int(mlp["router"]["top"])
+    idx, val = route(h, w[p + "mlp.router"], top)
     y = torch.zeros(h.shape[0], w[p + "mlp.e0.down"].shape[0], dtype=F64)
     lim = float(mlp["expert"]["limit"])
-    for t in range(h.shape[0]):
-        for e, s in zip(idx[t].tolist(), val[t].tolist()):
+    for j in range(top):                                   # the j-th choice of every token
+        for e in idx[:, j].unique().tolist():
+            rows = idx[:, j] == e
             q = f"{p}mlp.e{e}."
-            y[t] += clamped_glu(h[t:t + 1] * s, w[q + "gate"], w[q + "up"], w[q + "down"], lim)[0]
+            y[rows] += clamped_glu(h[rows] * val[rows, j:j + 1], w[q + "gate"], w[q + "up"], w[q + "down"], lim)
     sh = mlp.get("shared")
     if sh:
         q = p + "mlp.shared."

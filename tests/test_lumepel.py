@@ -85,7 +85,8 @@ def build(device, dtype="float32", seed=0, pages=24, seqs=4, cd=None, graphs=Non
     model = LumepelModel(cfg, device, tdt, weights=w)
     kw = dict(model="lumepel-test", dtype=dtype, max_num_seqs=seqs, max_batched_tokens=512, max_model_len=512,
               kv_cache_blocks=pages, detokenize=False, use_graphs=(device == "cuda") if graphs is None else graphs,
-              graph_batch_sizes=(1, 2, 4), mixed_graphs=False, logits_tap=True, tuned_gemms=False, async_decode=False)
+              graph_batch_sizes=(1, 2, 4), mixed_graphs=False, logits_tap=True, tuned_gemms=False, async_decode=False,
+              enable_prefix_caching=False)   # replayed rows bring every token themselves
     kw.update(eng)
     e = LLMEngine(EngineConfig(**kw), device=device, model=model)
     return e, cd, w
@@ -455,6 +456,19 @@ def test_preemption_recomputes(device):
     assert got == [r.output_ids for r in big.generate(prompts, sp)]
     assert got[0] == O.greedy(cd, W, prompts[0], 20)
     assert small.sched.free_blocks() == 5
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_prefix_cache_reuses_pages(device):
+    """A second request that starts with an earlier prompt takes its full pages from the prefix
+    cache (only the rest is prefilled) and generates what the oracle generates."""
+    eng, cd, W = build(device, "float32", enable_prefix_caching=True)
+    p = tokens(150, seed=3)
+    sp = SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True)
+    assert eng.generate([p], sp)[0].output_ids == O.greedy(cd, W, p, 8)
+    before = eng.stats["prefill_tokens"]
+    assert eng.generate([p + [5, 6, 7]], sp)[0].output_ids == O.greedy(cd, W, p + [5, 6, 7], 8)
+    assert eng.stats["prefill_tokens"] - before == 153 - 128 and eng.sched.prefix_hits() > 0
 
 
 def test_model_folder_roundtrip(tmp_path):
