@@ -227,7 +227,7 @@ def o_attention_in_keys(q, rows, dv, scale, pos):
 
 
 @pytest.mark.parametrize("shape", [(3, 26, 20), (18, 96, 64), (4, 192, 128), (2, 320, 256), (1, 13, 13), (2, 64, 32),
-                                   (3, 128, 64), (2, 256, 128), (1, 600, 530)])
+                                   (3, 128, 64), (2, 256, 128), (1, 600, 530), (3, 96, 64)])
 @pytest.mark.parametrize("device,dtype", DTYPES)
 def test_one_key_stands_out_and_random(device, dtype, shape):
     """Values read out of the key rows. One key row is made to match a scaled query, far back,
@@ -539,6 +539,22 @@ def test_mfma_forms_run_and_agree_with_the_plain_kernels():
     q = torch.randn(4, 192 * 4, generator=g).bfloat16().to(dev)
     assert ops.softmax_attention_mfma_ok(q, 192, 128, 4, 1) and ops.softmax_attention_mfma_ok(q, 96, 64, 8, 1)
     assert not ops.softmax_attention_mfma_ok(q, 112, 96, 4, 1)
+    # prompt portions of unequal length with earlier context: two heads per wave against one
+    Hh, Wk, dv, npg = 6, 192, 128, 40
+    page = (0.4 * torch.randn(npg, 1, 64, Wk, generator=g)).bfloat16().to(dev)
+    bt = torch.randperm(npg, generator=g).to(torch.int32).view(2, 20).to(dev)
+    cu = torch.tensor([0, 301, 370], dtype=torch.int32, device=dev)
+    ctx = torch.tensor([1000, 69], dtype=torch.int32, device=dev)
+    qq = torch.randn(370, Hh * Wk, generator=g).bfloat16().to(dev)
+    outs = []
+    for form in (0, 1):
+        with ops.kernel_forms(sm_share_heads=form):
+            outs.append(ops.softmax_attention_prefill(qq, page, page, bt, cu, ctx, 301, Hh, 1, Wk, dv, scale=0.07,
+                                                      v_in_k=True).float())
+    seq, pos = ops._rows_of_portions(cu, ctx, 370, dev)
+    want = ops.softmax_attention(qq, page, page, bt, seq, pos, Hh, 1, Wk, dv, scale=0.07, v_in_k=True).float()
+    for o in outs:
+        assert (o - want).abs().max().item() < 0.03 * max(1.0, want.abs().max().item())
 
 
 @pytest.mark.parametrize("device", DEVICES)
