@@ -258,8 +258,11 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
   extern __shared__ __attribute__((aligned(16))) uint16_t sm_lds[];
   uint16_t* k_s = sm_lds;                       // [KM][KT * DK]
   uint16_t* v_s = sm_lds + KM * KT * DK;        // [DV * KT]
-  // the last row blocks of a sequence see the most pages: they are launched first
-  const int tile = gridDim.x - 1 - blockIdx.x, hq = blockIdx.y, b = blockIdx.z;
+  // Longest first: the row block is the slowest grid index and counts down, so the blocks that
+  // see the most pages are dispatched first for every head and sequence, and the short ones fill
+  // the gaps at the end (with the row block as the fastest index the second half of the grid
+  // started its longest blocks late: the CUs were busy 56 % of a causal 8 x 2048-token launch).
+  const int tile = gridDim.z - 1 - blockIdx.z, hq = blockIdx.x, b = blockIdx.y;
   const int q0 = P.cu_q[b], qlen = P.cu_q[b + 1] - q0;
   if (tile * 64 >= qlen) return;
   const int ctx = P.ctx_lens[b];
@@ -304,8 +307,11 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
   // the current one is processed, so its latency hides behind the MFMA work.
   constexpr bool PREFETCH = (KM * PER_K + 4 * VBLK) * 4 <= 48;
   u16x8 kreg[KM][PER_K], vreg[VBLK][4];
-  auto fetch = [&](int t) {
-    const int64_t blk = P.block_tables[(int64_t)b * P.max_blocks + t];
+  // the page number of the next fetch is looked up one iteration ahead, so that the page loads do
+  // not wait for the table
+  const int32_t* btp = P.block_tables + (int64_t)b * P.max_blocks;
+  int blk_next = btp[t_first];
+  auto fetch = [&](int64_t blk) {
     const uint16_t* kp = P.kc + (blk * P.G + g) * (int64_t)(KM * KT * DK);
     const uint16_t* vp = P.vc + (blk * P.G + g) * (int64_t)KT * P.v_row;
 #pragma unroll
@@ -321,7 +327,8 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
       }
     }
   };
-  fetch(t_first);
+  fetch(blk_next);
+  if (t_first < t_last) blk_next = btp[t_first + 1];
   for (int t = t_first; t <= t_last; ++t) {
     __syncthreads();   // the previous page's reads are done
 #pragma unroll
@@ -351,7 +358,10 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
       }
     }
     __syncthreads();
-    if (PREFETCH && t < t_last) fetch(t + 1);
+    if (PREFETCH && t < t_last) {
+      fetch(blk_next);
+      if (t + 1 < t_last) blk_next = btp[t + 2];
+    }
 
     const int kbase = t * KT;
     const float fd = (float)(qpos - kbase - 8 * h);
@@ -441,7 +451,10 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
         for (int m = 0; m < MAPS; ++m) o[m][dt] = mfma16(a, pf[m][gg], o[m][dt]);
       }
     }
-    if (!PREFETCH && t < t_last) fetch(t + 1);
+    if (!PREFETCH && t < t_last) {
+      fetch(blk_next);
+      if (t + 1 < t_last) blk_next = btp[t + 2];
+    }
   }
   // lane (query col, h) holds value columns 16 dt + 4 h + rr of its query
   float inv[MAPS];
@@ -542,7 +555,7 @@ template <int DK, int DV>
 void launch_sm_mfma_shared(const SmMfmaParams& P, dim3 grid, hipStream_t stream) {
   constexpr size_t smem = (size_t)(64 * DK + DV * 64) * sizeof(uint16_t);
   static_assert(smem <= 65536, "dynamic LDS without the attribute");
-  grid.y = (unsigned)(P.H / 2);
+  grid.x = (unsigned)(P.H / 2);
   softmax_attention_mfma_kernel<DK, DV, 2, 2, true><<<grid, 256, smem, stream>>>(P);
 }
 
@@ -990,7 +1003,7 @@ void launch_softmax_attention_mfma(uint16_t* out, const uint16_t* q, int64_t q_s
   if (B == 0 || max_q_len == 0) return;
   SmMfmaParams P{out, q, gate, kc, vc, block_tables, cu_q, ctx_lens, q_stride, g_stride, max_blocks, H, G, window,
                  scale * 1.4426950408889634f, lam, unit_eps, out_scale, v_in_k ? dk : dv};
-  const dim3 grid((unsigned)((max_q_len + 63) / 64), (unsigned)H, (unsigned)B);
+  const dim3 grid((unsigned)H, (unsigned)B, (unsigned)((max_q_len + 63) / 64));   // (head, sequence, row block)
   const bool ok = maps == 2 ? launch_sm_mfma_dk<2>(P, dk, dv, grid, stream) : launch_sm_mfma_dk<1>(P, dk, dv, grid, stream);
   if (!ok) abort();   // the caller checks softmax_attention_mfma_supported
 }
