@@ -262,7 +262,9 @@ __global__ void __launch_bounds__(256) sigmoid_attention_mfma_kernel(const SigMf
   constexpr int SWS = NCH_K >= 16 ? 0 : NCH_K == 8 ? 1 : 2;
   __shared__ __attribute__((aligned(16))) uint16_t k_s[KT * DK];
   __shared__ __attribute__((aligned(16))) uint16_t v_s[DV * KT];
-  const int tile = blockIdx.x, hq = blockIdx.y, b = blockIdx.z;
+  // the row block is the slowest grid index and counts down: the blocks that see the most pages
+  // are dispatched first for every head and sequence
+  const int tile = gridDim.z - 1 - blockIdx.z, hq = blockIdx.x, b = blockIdx.y;
   const int q0 = P.cu_q[b], qlen = P.cu_q[b + 1] - q0;
   if (tile * 64 >= qlen) return;
   const int ctx = P.ctx_lens[b];
@@ -580,7 +582,7 @@ void launch_sigmoid_attention_mfma(uint16_t* out, const uint16_t* q, int64_t q_s
   if (B == 0 || max_q_len == 0) return;
   SigMfmaParams P{out, q, gate, kc, vc, block_tables, cu_q, ctx_lens, r1, r2, pb, q_stride, g_stride,
                   max_blocks, Hq, Hkv, window, keep_first, scale};
-  const dim3 grid((unsigned)((max_q_len + 63) / 64), (unsigned)Hq, (unsigned)B);
+  const dim3 grid((unsigned)Hq, (unsigned)B, (unsigned)((max_q_len + 63) / 64));   // (head, sequence, row block)
   bool ok = false;
   if (dk == 32) ok = launch_sig_mfma_dv<32>(P, dv, grid, stream);
   else if (dk == 64) ok = launch_sig_mfma_dv<64>(P, dv, grid, stream);
