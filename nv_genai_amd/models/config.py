@@ -774,3 +774,278 @@ def lumepel_layers(pattern: Sequence[str], hidden: int, heads: int, dim: int, ro
         blocks.append(LumepelLayer(t, m, mlp))
     return LumepelConfig(name=name, vocab_size=vocab_size, hidden=hidden, eps=eps, embed_scale=embed_scale,
                          logit_scale=logit_scale, logit_softcap=logit_softcap, blocks=tuple(blocks))
+
+
+# ---------------------------------------------------------------------------------------------
+# Lizezen: parallel layers behind one dynamic-tanh norm, mLSTM and rotary attention mixers, a
+# repeated span of layers with an input injection in front of every pass.
+@dataclass(frozen=True)
+class MlstmSpec:
+    """Mixer ``mlstm``: a matrix memory per head, ``S <- a S + b k v^T`` and a normaliser
+    ``n <- a n + b k`` with log-domain gates kept stable by a running maximum m; log input gate
+    ``cap tanh(z_i / cap)``, log forget gate ``logsigmoid(cap tanh(z_f / cap))``; every head's
+    output is brought to unit RMS, weighted, and gated by ``sigmoid(W_g h)``."""
+
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float
+
+
+@dataclass(frozen=True)
+class RotaryAttentionSpec:
+    """Mixers ``attention`` / ``attention_2``: causal softmax attention with GQA and rotary
+    positions (pairs (i, i + dims / 2)) on the first ``rot.dims`` elements of q and k heads.
+    ``qk_norm``: RMS norm of every q and k head (one weight of ``dim`` elements each) before the
+    rotation; ``values_from_keys``: the values are the key projections as they leave W_k (no
+    W_v; ``vdim`` = ``dim``); ``softcap`` > 0: scores go through ``softcap tanh(s / softcap)``;
+    ``head_gate``: every head's output is multiplied by ``sigmoid(W_g h)_head``."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    rot: RotarySpec
+    softcap: float = 0.0
+    qk_norm: bool = False
+    values_from_keys: bool = False
+    head_gate: bool = False
+
+
+@dataclass(frozen=True)
+class GeluMlpSpec:
+    """down(gelu_tanh(up x + b_up)) + b_down."""
+
+    ff: int
+    kind: str = "dense"
+
+
+@dataclass(frozen=True)
+class SwigluSpec:
+    """down(silu(gate x) * (up x)), no biases."""
+
+    ff: int
+
+
+@dataclass(frozen=True)
+class GroupedMoeSpec:
+    """``experts`` SwiGLU experts plus ``identity`` experts that return their input. Scores are a
+    softmax over all ``experts + identity`` router outputs; experts are chosen by score plus a
+    per-expert ``correction`` among the ``keep`` best of ``groups`` equal groups of neighbours (a
+    group's rank is its largest corrected score); the weights are the uncorrected scores of the
+    ``top`` chosen, divided by their sum, times ``scale``. ``shared``: an expert every token uses,
+    times ``sigmoid(sg . x)``."""
+
+    experts: int
+    top: int
+    expert: SwigluSpec
+    identity: int = 0
+    scale: float = 1.0
+    groups: int = 1
+    keep: int = 1
+    shared: Optional[SwigluSpec] = None
+    kind: str = "moe"
+
+    @property
+    def routed(self) -> int:
+        return self.experts + self.identity
+
+
+@dataclass(frozen=True)
+class LoopSpec:
+    """Layers ``start .. stop - 1`` run ``times`` times in a row with the same weights (every
+    pass with a cache / state of its own); in front of every pass the stream is replaced by
+    ``W_in [x ; x0]`` with x0 the embedding output."""
+
+    start: int
+    stop: int
+    times: int
+
+
+@dataclass(frozen=True)
+class LizezenLayer:
+    type: str                 # "mlstm" | "attention" | "attention_2"
+    mixer: object
+    mlp: object = None        # GeluMlpSpec | GroupedMoeSpec | None
+
+
+_LIZEZEN_MIXERS = ("mlstm", "attention", "attention_2")
+
+
+@dataclass(frozen=True)
+class LizezenConfig:
+    """Lizezen: parallel layers on an fp32 residual stream, ``h = dyt(x)``,
+    ``x += mixer(h) + ff(h)`` with ``dyt(x) = tanh(alpha x) * w + b`` (no statistics). Every size
+    and every constant that can differ between models comes from config.json
+    (:meth:`from_dict`)."""
+
+    name: str = "lizezen"
+    vocab_size: int = 512
+    hidden: int = 128
+    eps: float = 1e-5
+    blocks: tuple = ()
+    loop: Optional[LoopSpec] = None
+    max_position: int = 1 << 20     # no position table: only the engine's bookkeeping is bounded
+    arch: str = "lizezen"
+    bos_id: int = 0
+    eos_ids: tuple = ()
+    chat_format: str = "plain"
+
+    @property
+    def layers(self) -> int:
+        return len(self.blocks)
+
+    @property
+    def runs(self) -> tuple:
+        """The order the layers run in: ((layer index, first of a pass of the loop), ...)."""
+        n, lp = len(self.blocks), self.loop
+        if lp is None:
+            return tuple((i, False) for i in range(n))
+        out = [(i, False) for i in range(lp.start)]
+        for _ in range(lp.times):
+            out += [(i, i == lp.start) for i in range(lp.start, lp.stop)]
+        return tuple(out + [(i, False) for i in range(lp.stop, n)])
+
+    @property
+    def is_moe(self) -> bool:
+        return any(isinstance(b.mlp, GroupedMoeSpec) for b in self.blocks)
+
+    @property
+    def experts_per_tok(self) -> int:
+        """Largest top-k of any layer (sizes the engine's routing workspace)."""
+        return max([b.mlp.top for b in self.blocks if isinstance(b.mlp, GroupedMoeSpec)] or [1])
+
+    @property
+    def num_experts(self) -> int:
+        return max([b.mlp.experts for b in self.blocks if isinstance(b.mlp, GroupedMoeSpec)] or [0])
+
+    @staticmethod
+    def _rot(r: dict, what: str, dim: int) -> RotarySpec:
+        sc = r.get("scaling")
+        rot = RotarySpec(dims=int(r["dims"]), base=float(r["base"]), interleaved=False,
+                         yarn=None if not sc else (float(sc["factor"]), float(sc["original"]),
+                                                   float(sc["fast"]), float(sc["slow"])))
+        if rot.dims % 2 or not 0 < rot.dims <= dim:
+            raise ValueError(f"{what}: rot.dims must be even and at most dim")
+        return rot
+
+    @classmethod
+    def from_dict(cls, d: dict, name: str = "lizezen") -> "LizezenConfig":
+        blocks = []
+        for i, b in enumerate(d["layers"]):
+            t, m = b["type"], b["mixer"]
+            if t == "mlstm":
+                mixer = MlstmSpec(heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                                  gate_cap=float(m["gate_cap"]))
+                if not mixer.gate_cap > 0:
+                    raise ValueError(f"layer {i}: gate_cap must be positive")
+            elif t in ("attention", "attention_2"):
+                second = t == "attention_2"
+                dim = int(m["dim"])
+                mixer = RotaryAttentionSpec(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=dim,
+                                            vdim=int(m.get("vdim", dim)), scale=float(m["scale"]),
+                                            rot=cls._rot(m["rot"], f"layer {i}", dim),
+                                            softcap=float(m.get("softcap") or 0.0), qk_norm=second,
+                                            values_from_keys=second, head_gate=second)
+                if mixer.heads % mixer.kv_heads:
+                    raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+                if second and mixer.vdim != mixer.dim:
+                    raise ValueError(f"layer {i}: values taken from the keys need vdim = dim")
+            else:
+                raise ValueError(f"layer {i}: unknown mixer type {t!r} (known: {_LIZEZEN_MIXERS})")
+            if min(mixer.heads, mixer.dim, mixer.vdim) < 1:
+                raise ValueError(f"layer {i}: sizes must be positive")
+            mlp = b.get("mlp")
+            if mlp is not None:
+                kind = mlp.get("kind", "dense")
+                if kind == "dense":
+                    mlp = GeluMlpSpec(ff=int(mlp["ff"]))
+                elif kind == "moe":
+                    r, sh, g = mlp["router"], mlp.get("shared"), mlp["router"].get("groups")
+                    mlp = GroupedMoeSpec(experts=int(r["experts"]), top=int(r["top"]),
+                                         expert=SwigluSpec(int(mlp["expert"]["ff"])),
+                                         identity=int(r.get("identity") or 0), scale=float(r.get("scale", 1.0)),
+                                         groups=int(g["count"]) if g else 1, keep=int(g["keep"]) if g else 1,
+                                         shared=None if not sh else SwigluSpec(int(sh["ff"])))
+                    if mlp.routed % mlp.groups or not 1 <= mlp.keep <= mlp.groups:
+                        raise ValueError(f"layer {i}: {mlp.routed} routed outputs in {mlp.groups} groups, keep {mlp.keep}")
+                    if not 1 <= mlp.top <= mlp.keep * (mlp.routed // mlp.groups):
+                        raise ValueError(f"layer {i}: top {mlp.top} does not fit the kept groups")
+                else:
+                    raise ValueError(f"layer {i}: unknown feed-forward kind {kind!r}")
+            blocks.append(LizezenLayer(type=t, mixer=mixer, mlp=mlp))
+        lp = d.get("loop")
+        loop = None
+        if lp:
+            loop = LoopSpec(start=int(lp["start"]), stop=int(lp["stop"]), times=int(lp["times"]))
+            if not (0 <= loop.start < loop.stop <= len(blocks)) or loop.times < 1:
+                raise ValueError(f"loop {lp} does not fit {len(blocks)} layers")
+        return cls(name=name, vocab_size=int(d["vocab"]), hidden=int(d["width"]), eps=float(d["norm"]["eps"]),
+                   blocks=tuple(blocks), loop=loop)
+
+    def to_json_dict(self) -> dict:
+        """The config.json form (inverse of :meth:`from_dict`)."""
+        layers = []
+        for b in self.blocks:
+            m = b.mixer
+            if b.type == "mlstm":
+                mx = {"heads": m.heads, "dim": m.dim, "vdim": m.vdim, "gate_cap": m.gate_cap}
+            else:
+                rot = {"base": m.rot.base, "dims": m.rot.dims}
+                if m.rot.yarn:
+                    rot["scaling"] = dict(zip(("factor", "original", "fast", "slow"), m.rot.yarn))
+                mx = {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim, "vdim": m.vdim, "scale": m.scale, "rot": rot}
+                if m.softcap:
+                    mx["softcap"] = m.softcap
+            f = b.mlp
+            if isinstance(f, GroupedMoeSpec):
+                router = {"experts": f.experts, "top": f.top, "identity": f.identity, "scale": f.scale}
+                if f.groups > 1:
+                    router["groups"] = {"count": f.groups, "keep": f.keep}
+                ff = {"kind": "moe", "router": router, "expert": {"ff": f.expert.ff}}
+                if f.shared is not None:
+                    ff["shared"] = {"ff": f.shared.ff}
+            elif f is not None:
+                ff = {"kind": "dense", "ff": f.ff}
+            else:
+                ff = None
+            layers.append({"type": b.type, "mixer": mx, "mlp": ff})
+        out = {"architecture": "Lizezen", "vocab": self.vocab_size, "width": self.hidden, "norm": {"eps": self.eps},
+               "layers": layers}
+        if self.loop is not None:
+            out["loop"] = {"start": self.loop.start, "stop": self.loop.stop, "times": self.loop.times}
+        return out
+
+    def to_dict(self):
+        return asdict(self)
+
+
+def lizezen_layers(pattern: Sequence[str], hidden: int, heads: int, kv_heads: int, dim: int, vdim: int, ff: int,
+                   mlstm_heads: int = 0, mlstm_dim: int = 0, mlstm_vdim: int = 0, experts: int = 0, top: int = 2,
+                   expert_ff: int = 0, shared_ff: int = 0, identity: int = 0, groups: int = 1, keep: int = 1,
+                   route_scale: float = 1.0, softcap: float = 0.0, gate_cap: float = 15.0, rot_base: float = 10000.0,
+                   rot_dims: int = 0, yarn: Optional[tuple] = None, loop: Optional[tuple] = None,
+                   vocab_size: int = 32768, eps: float = 1e-5, name: str = "lizezen") -> LizezenConfig:
+    """A Lizezen config from a pattern of mixer types with the same sizes in every layer of a
+    kind (benchmarks, tests). ``experts`` > 0: every second feed-forward is a mixture (the others
+    dense of ``ff``; ``ff`` 0: none). ``loop`` = (start, stop, times)."""
+    blocks = []
+    for i, t in enumerate(pattern):
+        if t == "mlstm":
+            m = MlstmSpec(mlstm_heads or heads, mlstm_dim or dim, mlstm_vdim or vdim, gate_cap)
+        elif t in ("attention", "attention_2"):
+            second = t == "attention_2"
+            rot = RotarySpec(rot_dims or dim, rot_base, False, yarn if second else None)
+            m = RotaryAttentionSpec(heads, heads if second else kv_heads, dim, dim if second else vdim, dim ** -0.5, rot,
+                                    softcap if second else 0.0, second, second, second)
+        else:
+            raise ValueError(f"unknown mixer type {t!r}")
+        if experts and i % 2:
+            mlp = GroupedMoeSpec(experts, top, SwigluSpec(expert_ff), identity, route_scale, groups, keep,
+                                 SwigluSpec(shared_ff) if shared_ff else None)
+        else:
+            mlp = GeluMlpSpec(ff) if ff else None
+        blocks.append(LizezenLayer(t, m, mlp))
+    return LizezenConfig(name=name, vocab_size=vocab_size, hidden=hidden, eps=eps, blocks=tuple(blocks),
+                         loop=None if not loop else LoopSpec(*loop))

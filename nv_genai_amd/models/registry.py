@@ -14,7 +14,7 @@ from typing import Callable, Dict, Optional, Tuple
 
 import torch
 
-from .config import LLAMA_PRESETS, BidasunConfig, BiruvikConfig, LlamaConfig, LumepelConfig
+from .config import LLAMA_PRESETS, BidasunConfig, BiruvikConfig, LizezenConfig, LlamaConfig, LumepelConfig
 
 # design name (lower case) -> (config builder from the config.json dict, model class loader)
 _REGISTRY: Dict[str, Tuple[Callable[[dict], object], Callable[[], type]]] = {}
@@ -40,6 +40,12 @@ def _lumepel_class():
     from .lumepel import LumepelModel
 
     return LumepelModel
+
+
+def _lizezen_class():
+    from .lizezen import LizezenModel
+
+    return LizezenModel
 
 
 def _llama_class():
@@ -80,6 +86,7 @@ def _hf_decoder_config(d: dict) -> LlamaConfig:
 register("bidasun", BidasunConfig.from_dict, _bidasun_class)
 register("biruvik", BiruvikConfig.from_dict, _biruvik_class)
 register("lumepel", LumepelConfig.from_dict, _lumepel_class)
+register("lizezen", LizezenConfig.from_dict, _lizezen_class)
 for _t in _HF_ARCH:
     register(_t, _hf_decoder_config, _llama_class)
 
@@ -92,6 +99,8 @@ def model_class_for(cfg) -> type:
         return _biruvik_class()
     if isinstance(cfg, LumepelConfig):
         return _lumepel_class()
+    if isinstance(cfg, LizezenConfig):
+        return _lizezen_class()
     if isinstance(cfg, LlamaConfig):
         return _llama_class()
     raise ValueError(f"no model class for {type(cfg).__name__}")

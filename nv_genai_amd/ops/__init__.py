@@ -7,7 +7,7 @@ GPU call raises (so a GPU test can never pass on an eager-PyTorch substitute).
 from __future__ import annotations
 
 import contextlib
-
+import math
 from typing import Optional, Tuple
 
 import torch
@@ -502,13 +502,18 @@ def softcap_(z: torch.Tensor, cap: float) -> torch.Tensor:
     return z
 
 
-def group_rmsnorm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float, dtype: torch.dtype) -> torch.Tensor:
-    """RMS norm of each of ``groups`` equal column groups of fp32 rows (one weight per element of
-    a group, shared by the groups), written in ``dtype``."""
+def group_rmsnorm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float, dtype: torch.dtype,
+                  gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """RMS norm of each of ``groups`` equal column groups of fp32 rows, written in ``dtype``. ``w``
+    (fp32) holds one weight per element of a group, shared by the groups, or one per column of the
+    row. ``gate`` [T, columns] (rows of the activation type, any row stride): the result is
+    multiplied by ``sigmoid(gate)``."""
+    if w.numel() not in (x.shape[1] // groups, x.shape[1]):
+        raise ValueError("group_rmsnorm: one weight per group element or per column")
     if not _gpu(x):
-        return ref.group_rmsnorm(x, w, groups, eps, dtype)
+        return ref.group_rmsnorm(x, w, groups, eps, dtype, gate)
     out = torch.empty(x.shape, dtype=dtype, device=x.device)
-    kernels().group_rmsnorm(out, x, w, int(groups), float(eps))
+    kernels().group_rmsnorm(out, x, w, int(groups), float(eps), gate)
     return out
 
 
@@ -531,7 +536,7 @@ def headnorm_cache_(proj, slots, kc, vc, nq: int, nk: int, dk: int, nv: int, dv:
 
 def softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H: int, G: int, dk: int, dv: int, scale: float,
                       window: int = 0, maps: int = 1, lam: float = 0.0, unit_eps: Optional[float] = None,
-                      out_scale: float = 1.0, gate=None, out=None, v_in_k: bool = False):
+                      out_scale: float = 1.0, gate=None, out=None, v_in_k: bool = False, softcap: float = 0.0):
     """Softmax attention of token rows (prompt portions and single-token rows alike) over row-
     major pages K [blocks, G * maps, 64, dk], V [blocks, G, 64, dv]. The query at position i
     sees keys ``j <= i`` (``window`` > 0: and ``i - j < window``). ``maps`` (1 or 2) score maps per
@@ -542,17 +547,19 @@ def softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H: int, G: int, dk:
     head outputs are multiplied by ``sigmoid(gate)``. ``tok_seq[t]`` is the block-table row of
     token t, ``pos[t]`` its position (negative: padding row, zeros out). Scores, softmax and
     accumulation are fp32. ``v_in_k`` (one map, dv <= dk): the values are the first dv elements of
-    the key rows (``vc`` is not read) - keys with extra key-only columns behind a shared latent."""
+    the key rows (``vc`` is not read) - keys with extra key-only columns behind a shared latent.
+    ``softcap`` > 0: a score s becomes ``softcap * tanh(s / softcap)`` before the softmax."""
     if v_in_k and (maps != 1 or dv > dk):
         raise ValueError("values inside the key rows: one map and dv <= dk")
     if not _gpu(q):
         return ref.softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv, scale, window, maps, lam,
-                                     unit_eps, out_scale, gate, v_in_k)
+                                     unit_eps, out_scale, gate, v_in_k, softcap)
     if out is None:
         out = torch.empty(q.shape[0], H * dv, dtype=q.dtype, device=q.device)
     kernels().softmax_attention(out, q, gate, kc, kc if v_in_k else vc, block_tables, tok_seq, pos, H, G, dk, dv,
                                 float(scale), int(window), int(maps), float(lam),
-                                -1.0 if unit_eps is None else float(unit_eps), float(out_scale), bool(v_in_k))
+                                -1.0 if unit_eps is None else float(unit_eps), float(out_scale), bool(v_in_k),
+                                float(softcap))
     return out
 
 
@@ -576,28 +583,29 @@ def _rows_of_portions(cu_q, ctx_lens, T: int, dev):
 def softmax_attention_prefill(q, kc, vc, block_tables, cu_q, ctx_lens, max_q_len: int, H: int, G: int, dk: int,
                               dv: int, scale: float, window: int = 0, maps: int = 1, lam: float = 0.0,
                               unit_eps: Optional[float] = None, out_scale: float = 1.0, gate=None, out=None,
-                              v_in_k: bool = False):
+                              v_in_k: bool = False, softcap: float = 0.0):
     """:func:`softmax_attention` of prompt portions on MFMA tiles: sequence b owns token rows
     ``[cu_q[b], cu_q[b + 1])``, the last ones of its ``ctx_lens[b]`` keys. Rows the tile kernel
     does not take (fp32, other head sizes, CPU) run the row form."""
     if not softmax_attention_mfma_ok(q, dk, dv, H // G, maps):
         seq, pos = _rows_of_portions(cu_q, ctx_lens, q.shape[0], q.device)
         return softmax_attention(q, kc, vc, block_tables, seq, pos, H, G, dk, dv, scale, window, maps, lam, unit_eps,
-                                 out_scale, gate, out=out, v_in_k=v_in_k)
+                                 out_scale, gate, out=out, v_in_k=v_in_k, softcap=softcap)
     if v_in_k and (maps != 1 or dv > dk):
         raise ValueError("values inside the key rows: one map and dv <= dk")
     if out is None:
         out = torch.empty(q.shape[0], H * dv, dtype=q.dtype, device=q.device)
     kernels().softmax_attention_prefill(out, q, gate, kc, kc if v_in_k else vc, block_tables, cu_q, ctx_lens,
                                         int(max_q_len), H, G, dk, dv, float(scale), int(window), int(maps), float(lam),
-                                        -1.0 if unit_eps is None else float(unit_eps), float(out_scale), bool(v_in_k))
+                                        -1.0 if unit_eps is None else float(unit_eps), float(out_scale), bool(v_in_k),
+                                        float(softcap))
     return out
 
 
 def softmax_attention_rows(q, kc, vc, block_tables, tok_seq, pos, H: int, G: int, dk: int, dv: int, scale: float,
                            max_ctx: int, window: int = 0, maps: int = 1, lam: float = 0.0,
                            unit_eps: Optional[float] = None, out_scale: float = 1.0, gate=None, out=None,
-                           v_in_k: bool = False):
+                           v_in_k: bool = False, softcap: float = 0.0):
     """:func:`softmax_attention` of single-token rows (decode rows; any rows work) on the page-
     parallel MFMA kernel: the query heads that share a KV head are the columns of one tile, so a
     page is read once per group; the visible pages of a row are split over several workgroups
@@ -605,7 +613,7 @@ def softmax_attention_rows(q, kc, vc, block_tables, tok_seq, pos, H: int, G: int
     normalises and gates. ``max_ctx`` bounds the rows' positions (launch shape)."""
     if not softmax_attention_mfma_ok(q, dk, dv, H // G, maps):
         return softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv, scale, window, maps, lam,
-                                 unit_eps, out_scale, gate, out=out, v_in_k=v_in_k)
+                                 unit_eps, out_scale, gate, out=out, v_in_k=v_in_k, softcap=softcap)
     if v_in_k and (maps != 1 or dv > dk):
         raise ValueError("values inside the key rows: one map and dv <= dk")
     C = kernels()
@@ -616,7 +624,8 @@ def softmax_attention_rows(q, kc, vc, block_tables, tok_seq, pos, H: int, G: int
         out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
     C.softmax_attention_decode(out, ws, parts, q, gate, kc, kc if v_in_k else vc, block_tables, tok_seq, pos, H, G, dk,
                                dv, float(scale), int(window), int(maps), float(lam),
-                               -1.0 if unit_eps is None else float(unit_eps), float(out_scale), bool(v_in_k))
+                               -1.0 if unit_eps is None else float(unit_eps), float(out_scale), bool(v_in_k),
+                               float(softcap))
     return out
 
 
@@ -692,14 +701,16 @@ def latent_rope_cache_(proj, pos, slots, page, freq, mag: float, interleaved: bo
     return proj
 
 
-def clamped_glu(x: torch.Tensor, F: int, limit: float, alpha: float = 1.702, gate_col: int = -1) -> torch.Tensor:
-    """Rows ``[gate F | up F | ...]`` -> ``g * sigmoid(alpha g) * (u + 1)`` [T, F] with
+def clamped_glu(x: torch.Tensor, F: int, limit: float, alpha: float = 1.702, gate_col: int = -1,
+                shift: float = 1.0) -> torch.Tensor:
+    """Rows ``[gate F | up F | ...]`` -> ``g * sigmoid(alpha g) * (u + shift)`` [T, F] with
     ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``; ``gate_col`` >= 0: times
-    ``sigmoid(x[:, gate_col])`` (one gate per row). fp32 math, bf16 or fp32 rows, any F."""
+    ``sigmoid(x[:, gate_col])`` (one gate per row). ``limit = inf, alpha = 1, shift = 0`` is
+    SwiGLU. fp32 math, bf16 or fp32 rows, any F."""
     if not _gpu(x):
-        return ref.clamped_glu(x, F, limit, alpha, gate_col)
+        return ref.clamped_glu(x, F, limit, alpha, gate_col, shift)
     out = torch.empty(x.shape[0], F, dtype=x.dtype, device=x.device)
-    kernels().clamped_glu(out, x, int(F), float(limit), float(alpha), int(gate_col))
+    kernels().clamped_glu(out, x, int(F), float(limit), float(alpha), int(gate_col), float(shift))
     return out
 
 
@@ -711,6 +722,73 @@ def scale_softcap_(z: torch.Tensor, scale: float, cap: float) -> torch.Tensor:
         kernels().softcap(z, float(cap), float(scale))
         return z
     return z.mul_(scale) if scale != 1.0 else z
+
+
+# ------------------------------------------------------------------------- dynamic-tanh stream, rotary attention with head norms
+def dyt_norm(x: torch.Tensor, alpha: float, w: torch.Tensor, b: torch.Tensor, rows: Optional[torch.Tensor] = None,
+             dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """Dynamic tanh in place of a norm: ``tanh(alpha x) * w + b`` of fp32 rows (``rows``: only
+    these), no statistics, written in ``dtype``. ``w``, ``b`` fp32 [columns]."""
+    if not _gpu(x):
+        return ref.dyt_norm(x, alpha, w, b, rows, dtype)
+    n = x.shape[0] if rows is None else rows.numel()
+    out = torch.empty(n, x.shape[1], dtype=dtype, device=x.device)
+    kernels().dyt_norm(out, x, float(alpha), w, b, rows)
+    return out
+
+
+def residual_dyt_(x: torch.Tensor, y1: torch.Tensor, y2: Optional[torch.Tensor], bias: Optional[torch.Tensor],
+                  norm: Optional[tuple], dtype: torch.dtype, assign: bool = False) -> Optional[torch.Tensor]:
+    """Step of a parallel layer on an fp32 stream, one launch: ``x += (y1 + y2 + bias)`` in place
+    (the two sub-layer outputs and an fp32 bias row are summed first, in fp32), or ``x = y1`` when
+    ``assign`` (a projection replaces the stream). ``norm`` = (alpha, w, b): also returns
+    ``tanh(alpha x) * w + b`` in ``dtype`` (the next layer's input); None: returns None."""
+    out = None if norm is None else torch.empty(x.shape, dtype=dtype, device=x.device)
+    if not _gpu(x):
+        ref.residual_dyt_(x, y1, y2, bias, norm, out, assign)
+        return out
+    a, w, b = norm if norm is not None else (0.0, None, None)
+    kernels().residual_dyt(x, y1, y2, bias, float(a), w, b, out, bool(assign))
+    return out
+
+
+def pack_pair(a: torch.Tensor, b: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """Rows ``[a | b]`` of two fp32 streams in ``dtype`` (the input of a projection that mixes the
+    stream with the embedding output)."""
+    if not _gpu(a):
+        return ref.pack_pair(a, b, dtype)
+    out = torch.empty(a.shape[0], a.shape[1] + b.shape[1], dtype=dtype, device=a.device)
+    kernels().pack_pair(out, a, b)
+    return out
+
+
+def bias_gelu_tanh_(x: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """``x = gelu_tanh(x + bias)`` in place: rows of any width, bf16 or fp32, fp32 bias and math."""
+    if not _gpu(x):
+        return ref.bias_gelu_tanh_(x, bias)
+    kernels().bias_gelu_tanh(x, bias)
+    return x
+
+
+def rope_headnorm_cache_(proj, pos, slots, kc, vc, H: int, G: int, dk: int, dv: int, freq, mag: float, rot_dims: int,
+                         eps: float, q_w=None, k_w=None, v_off: Optional[int] = None):
+    """Projection rows ``[q: H heads of dk | k: G heads of dk | ...]`` in place, one launch:
+    RMS-normalise every q head with ``q_w`` [dk] and every k head with ``k_w`` [dk] (None: left
+    as it is), then rotary positions on the first ``rot_dims`` elements of every q and k head
+    (pair i = elements (i, i + rot_dims / 2) at angle ``pos * freq[i]`` - float64 product reduced
+    to one turn before the fp32 cos / sin -, cos and sin times ``mag``), q and k written back, k
+    into the token's page slot of K [blocks, G, 64, dk]. The values go into V [blocks, G, 64, dv]:
+    columns ``v_off .. v_off + G * dv`` of the row, or, with ``v_off`` None (dv = dk), the k heads
+    as projected, before norm and rotation. ``slots`` < 0: no page write. Norms and rotation fp32."""
+    if rot_dims % 2 or rot_dims > dk or freq.numel() != rot_dims // 2:
+        raise ValueError("rotary positions: an even number of elements, at most the head size")
+    if v_off is None and dv != dk:
+        raise ValueError("values taken from the keys need dv = dk")
+    if not _gpu(proj):
+        return ref.rope_headnorm_cache_(proj, pos, slots, kc, vc, H, G, dk, dv, freq, mag, rot_dims, eps, q_w, k_w, v_off)
+    kernels().rope_headnorm_cache(proj, pos, slots, kc, vc, int(H), int(G), int(dk), int(dv), freq, float(mag),
+                                  int(rot_dims), float(eps), q_w, k_w, -1 if v_off is None else int(v_off))
+    return proj
 
 
 # ------------------------------------------------------------------------- gated linear recurrence
@@ -726,6 +804,32 @@ def hgrn2_scan(proj, f_bias, lower, state, H: int, d: int, dv: int, cu, slots, p
         return ref.hgrn2_scan(proj, f_bias, lower, state, H, d, dv, cu, slots, pos)
     out = torch.empty(proj.shape[0], H * dv, dtype=torch.float32, device=proj.device)
     kernels().hgrn2_scan(out, proj, f_bias, lower, state, H, d, dv, cu, slots, pos)
+    return out
+
+
+def mlstm_state_size(d: int, dv: int) -> int:
+    """fp32 elements of one head's mLSTM state: S [d, dv], n [d], m."""
+    return d * dv + d + 1
+
+
+def mlstm_scan(proj, gate_bias, state, H: int, d: int, dv: int, cap: float, cu, slots, pos, offs) -> torch.Tensor:
+    """mLSTM recurrence (matrix memory with exponential gates) over a step's rows. ``offs`` =
+    (q, k, v, gates) column offsets in ``proj``: q and k [H*d], v [H*dv], and 2H gate
+    pre-activations ``[i (H) | f (H)]``. In fp32: ``q *= d^-0.5``,
+    ``i = cap tanh((i + b_i) / cap)``, ``f = logsigmoid(cap tanh((f + b_f) / cap))`` with
+    ``gate_bias`` = [b_i | b_f]; per row ``m' = max(f + m, i)``,
+    ``S <- e^(f + m - m') S + e^(i - m') k v^T``, ``n`` likewise with k alone,
+    ``o = S^T q / (max(|n . q|, e^(-m')) + 1e-6)``. Segment b is rows ``cu[b] .. cu[b + 1]``
+    (``cu`` None: row b alone) of one sequence; its state (S, n, m) comes from ``state[slots[b]]``
+    ([slots, H, d * dv + d + 1] fp32), or zeros (m = 0) when the segment starts at position 0 - a
+    reused slot needs no clearing - and goes back there. ``slots[b]`` < 0: nothing is read or
+    kept. Returns the fp32 outputs [T, H*dv]."""
+    if not _gpu(proj):
+        return ref.mlstm_scan(proj, gate_bias, state, H, d, dv, cap, cu, slots, pos, offs)
+    out = torch.empty(proj.shape[0], H * dv, dtype=torch.float32, device=proj.device)
+    q_off, k_off, v_off, g_off = (int(o) for o in offs)
+    kernels().mlstm_scan(out, proj, gate_bias, state, int(H), int(d), int(dv), float(cap), cu, slots, pos, q_off, k_off,
+                         v_off, g_off)
     return out
 
 
@@ -1042,6 +1146,30 @@ def moe_route_scores(logits: torch.Tensor, k: int, score: str = "sigmoid", renor
     return ids, w
 
 
+def moe_route_grouped(logits: torch.Tensor, correction: torch.Tensor, k: int, groups: int = 1, keep: int = 1,
+                      scale: float = 1.0, ws: Optional["MoEWorkspace"] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Group-limited routing from fp32 logits [T, E]: scores ``s = softmax(logits)`` over all E;
+    experts are chosen by ``s + correction`` (fp32 [E]) among the ``keep`` of ``groups`` equal
+    groups of neighbouring experts whose largest corrected score is largest (the others cannot be
+    chosen, however their corrected scores compare); the ``k`` chosen (ties: the lower index) get
+    the weights ``s / (sum of the chosen s + 1e-20) * scale``. ids int32 [T, k], weights fp32
+    [T, k]. ``groups = 1``: plain top-k by corrected score."""
+    T, E = logits.shape
+    if logits.dtype != torch.float32 or correction.dtype != torch.float32 or correction.numel() != E:
+        raise ValueError("router logits and the correction are fp32, one correction per expert")
+    if groups < 1 or E % groups or not 1 <= keep <= groups or not 1 <= k <= keep * (E // groups):
+        raise ValueError(f"{E} experts in {groups} groups, keep {keep}, top {k}")
+    if not _gpu(logits):
+        return ref.moe_route_grouped(logits, correction, k, groups, keep, scale)
+    if ws is not None and ws.rows * ws.k >= T * k:
+        ids, w = ws.ids[:T * k].view(T, k), ws.w[:T * k].view(T, k)
+    else:
+        ids = torch.empty(T, k, dtype=torch.int32, device=logits.device)
+        w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+    kernels().moe_route_grouped(logits, correction, int(k), int(groups), int(keep), float(scale), ids, w)
+    return ids, w
+
+
 def moe_mfma_ok(x: torch.Tensor, F: int) -> bool:
     """The grouped MFMA GEMMs take bf16 rows with width % 256 == 0 and expert ff % 128 == 0."""
     return _gpu(x) and x.dtype == torch.bfloat16 and x.shape[1] % 256 == 0 and F % 128 == 0
@@ -1049,21 +1177,24 @@ def moe_mfma_ok(x: torch.Tensor, F: int) -> bool:
 
 def moe_glu_experts(x: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor,
                     limit: float, alpha: float = 1.702, weight_input: bool = True, add: Optional[torch.Tensor] = None,
-                    ws: Optional["MoEWorkspace"] = None) -> torch.Tensor:
+                    ws: Optional["MoEWorkspace"] = None, shift: float = 1.0, identity: bool = False) -> torch.Tensor:
     """Routed clamped-GLU experts on rows x [T, H] -> [T, H]: the sum over a row's experts
-    (``ids`` / ``wts`` [T, k] from :func:`moe_route_scores`) of
-    ``down_e(g * sigmoid(alpha g) * (u + 1))``, ``g = min(gate_e(s x), limit)``,
+    (``ids`` / ``wts`` [T, k] from :func:`moe_route_scores` / :func:`moe_route_grouped`) of
+    ``down_e(g * sigmoid(alpha g) * (u + shift))``, ``g = min(gate_e(s x), limit)``,
     ``u = clamp(up_e(s x), -limit, limit)`` with the routing weight on the expert's input
     (``weight_input``; else ``s = 1`` and the weight multiplies the expert's output). ``w13``
     [E, 2F, H] = [gate | up] rows per expert, ``w2`` [E, H, F]. ``add`` [T, H]: added to the sum in
-    the combining kernel (a shared expert's output).
+    the combining kernel (a shared expert's output). ``limit = inf, alpha = 1, shift = 0`` with the
+    weight on the output is a SwiGLU expert. ``identity``: ids >= E are experts that return their
+    input (``weight * x``, added by the combining kernel; they take no GEMM rows).
 
     GPU: ``moe_align`` (tokens sorted by expert, M-tile table) -> grouped gate|up GEMM with the
     weight and the activation in its epilogue -> grouped down GEMM -> combine (fp32 sum per token).
     bf16 rows with MFMA-sized experts run the grouped MFMA GEMMs, everything else (fp32, other
     sizes) a tiled fp32-accumulating kernel of the same structure."""
+    swiglu = math.isinf(limit) and alpha == 1.0 and shift == 0.0 and not weight_input
     if not _gpu(x):
-        return ref.moe_glu_experts(x, ids, wts, w13, w2, limit, alpha, weight_input, add)
+        return ref.moe_glu_experts(x, ids, wts, w13, w2, limit, alpha, weight_input, add, shift, identity)
     C = kernels()
     T, H = x.shape
     E, F2, K = w13.shape
@@ -1077,21 +1208,28 @@ def moe_glu_experts(x: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w13: 
     if ws.rows * ws.k < M or ws.E < E:
         raise ValueError(f"MoE workspace for {ws.rows} rows x top-{ws.k} / {ws.E} experts cannot take "
                          f"{T} rows x top-{k} / {E} experts")
-    mfma = moe_mfma_ok(x, F)
+    mfma = moe_mfma_ok(x, F) and (swiglu or shift == 1.0)
     bm = 64 if (not mfma or M <= 256 * E) else 128
     mt = -(-M // bm) + E
     C.moe_align(ids.reshape(-1), wts.reshape(-1), T, int(k), 0, E, bm, ws.sorted_tok, ws.sorted_w, ws.inv, ws.tiles, mt)
     h = torch.empty(M, F, dtype=x.dtype, device=x.device)
     y = torch.empty(M, H, dtype=x.dtype, device=x.device)
-    if mfma:
+    if mfma and swiglu:     # the silu epilogue of the Mixtral experts, weight on the down GEMM
+        C.moe_gemm(x, w13, ws.sorted_tok, ws.sorted_w, ws.tiles, mt, bm, h, 0, 0, 0.0, 0.0, False)
+        C.moe_gemm(h, w2, ws.sorted_tok, ws.sorted_w, ws.tiles, mt, bm, y, 1, 0, 0.0, 0.0, False)
+    elif mfma:
         C.moe_gemm(x, w13, ws.sorted_tok, ws.sorted_w, ws.tiles, mt, bm, h, 0, 2, float(limit), float(alpha),
                    bool(weight_input))
         C.moe_gemm(h, w2, ws.sorted_tok, ws.sorted_w, ws.tiles, mt, bm, y, 1, 0, 0.0, 0.0, bool(weight_input))
     else:
-        C.moe_gemm_rows(x, w13, ws.sorted_tok, ws.sorted_w, ws.tiles, mt, h, 0, float(limit), float(alpha),
-                        bool(weight_input))
-        C.moe_gemm_rows(h, w2, ws.sorted_tok, ws.sorted_w, ws.tiles, mt, y, 1, 0.0, 0.0, not weight_input)
-    C.moe_combine_rows(y, ws.inv, T, int(k), add, out)
+        lim = float(min(limit, 3.0e38))
+        C.moe_gemm_rows(x, w13, ws.sorted_tok, ws.sorted_w, ws.tiles, mt, h, 0, lim, float(alpha),
+                        bool(weight_input), float(shift))
+        C.moe_gemm_rows(h, w2, ws.sorted_tok, ws.sorted_w, ws.tiles, mt, y, 1, 0.0, 0.0, not weight_input, 0.0)
+    if identity:
+        C.moe_combine_rows(y, ws.inv, T, int(k), add, out, x, ids.reshape(-1), wts.reshape(-1), E)
+    else:
+        C.moe_combine_rows(y, ws.inv, T, int(k), add, out, None, None, None, E)
     return out
 
 

@@ -578,12 +578,12 @@ def headnorm_cache_(proj, slots, kc, vc, nq, nk, dk, nv, dv, eps, q_w=None, k_w=
 
 
 def softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv, scale, window=0, maps=1, lam=0.0,
-                      unit_eps=None, out_scale=1.0, gate=None, v_in_k=False):
+                      unit_eps=None, out_scale=1.0, gate=None, v_in_k=False, softcap=0.0):
     """Softmax attention of token rows over row-major pages, one row at a time. ``maps`` score
     maps per head (q head (h, m) at column (h * maps + m) * dk, k head (h // (H / G)) * maps + m,
     v head h // (H / G)), combined as a_0 - lam * a_1; optional unit RMS per head (times
     ``out_scale``) and a per-head sigmoid gate. ``v_in_k``: the values are the first dv elements
-    of the key rows."""
+    of the key rows. ``softcap`` > 0: scores become softcap * tanh(score / softcap)."""
     T = q.shape[0]
     out = torch.zeros(T, H, dv, dtype=torch.float32, device=q.device)
     BS = kc.shape[2]
@@ -601,6 +601,8 @@ def softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv, scale
         k = kc[blk, :, off, :].float().view(-1, G, maps, dk)[:, vh]     # [n, H, maps, dk]
         v = (kc[blk, :, off, :dv] if v_in_k else vc[blk, :, off, :]).float()[:, vh]   # [n, H, dv]
         s = torch.einsum("hmd,nhmd->hmn", qf[t], k) * scale
+        if softcap > 0:
+            s = softcap * torch.tanh(s / softcap)
         a = torch.einsum("hmn,nhd->hmd", torch.softmax(s, -1), v)
         out[t] = a[:, 0] - lam * a[:, 1] if maps == 2 else a[:, 0]
     if unit_eps is not None:
@@ -640,12 +642,17 @@ def hgrn2_scan(proj, f_bias, lower, state, H, d, dv, cu, slots, pos):
     return out.reshape(T, H * dv)
 
 
-def group_rmsnorm(x, w, groups, eps, dtype):
+def group_rmsnorm(x, w, groups, eps, dtype, gate=None):
     """RMS norm of every one of ``groups`` equal column groups of fp32 rows, weight per element
-    of a group, written in ``dtype``."""
+    of a group (or per column of the row), written in ``dtype``; ``gate`` [T, columns]: times
+    sigmoid(gate)."""
     T = x.shape[0]
     xg = x.view(T, groups, -1)
-    return (xg * torch.rsqrt(xg.pow(2).mean(-1, keepdim=True) + eps) * w).reshape(T, -1).to(dtype)
+    y = xg * torch.rsqrt(xg.pow(2).mean(-1, keepdim=True) + eps) * w.view(-1, xg.shape[2])
+    y = y.reshape(T, -1)
+    if gate is not None:
+        y = y * torch.sigmoid(gate.float())
+    return y.to(dtype)
 
 
 # ------------------------------------------------------------------------- pre-norm fp32 stream, rotated latent
@@ -707,13 +714,13 @@ def latent_rope_cache_(proj, pos, slots, page, freq, mag, interleaved, rot_dims,
     return proj
 
 
-def clamped_glu(x, F, limit, alpha, gate_col=-1):
-    """Rows [gate F | up F | ...] -> g * sigmoid(alpha g) * (u + 1), g = min(gate, limit),
+def clamped_glu(x, F, limit, alpha, gate_col=-1, shift=1.0):
+    """Rows [gate F | up F | ...] -> g * sigmoid(alpha g) * (u + shift), g = min(gate, limit),
     u = clamp(up, +-limit); times sigmoid(x[:, gate_col]) when gate_col >= 0."""
     xf = x.float()
     g = xf[:, :F].clamp(max=limit)
     u = xf[:, F:2 * F].clamp(min=-limit, max=limit)
-    y = g * torch.sigmoid(alpha * g) * (u + 1.0)
+    y = g * torch.sigmoid(alpha * g) * (u + shift)
     if gate_col >= 0:
         y = y * torch.sigmoid(xf[:, gate_col:gate_col + 1])
     return y.to(x.dtype)
@@ -733,10 +740,11 @@ def moe_route_scores(logits, k, score="sigmoid", renorm=False):
     return ids.to(torch.int32), w
 
 
-def moe_glu_experts(x, ids, wts, w13, w2, limit, alpha, weight_input=True, add=None):
+def moe_glu_experts(x, ids, wts, w13, w2, limit, alpha, weight_input=True, add=None, shift=1.0, identity=False):
     """Sum over a row's experts e of expert_e(x) with the routing weight on the expert's input
     (``weight_input``) or on its output; expert = clamped GLU, ``w13`` [E, 2F, H] = [gate | up],
-    ``w2`` [E, H, F]. ``add`` [T, H] is added to the sum."""
+    ``w2`` [E, H, F]. ``add`` [T, H] is added to the sum. ``identity``: ids >= E return the row
+    itself times the weight."""
     E, F2, _ = w13.shape
     F = F2 // 2
     out = torch.zeros(x.shape[0], w2.shape[1], dtype=torch.float32, device=x.device)
@@ -746,9 +754,130 @@ def moe_glu_experts(x, ids, wts, w13, w2, limit, alpha, weight_input=True, add=N
             continue
         wt = wts[tok, slot].unsqueeze(1)
         gu = (x[tok].float() @ w13[e].float().t()) * (wt if weight_input else 1.0)
-        h = clamped_glu(gu, F, limit, alpha).to(x.dtype)
+        h = clamped_glu(gu, F, limit, alpha, shift=shift).to(x.dtype)
         y = h.float() @ w2[e].float().t()
         out.index_add_(0, tok, y if weight_input else y * wt)
+    if identity:
+        out = out + x.float() * (wts * (ids >= E)).sum(-1, keepdim=True)
     if add is not None:
         out = out + add.float()
     return out.to(x.dtype)
+
+
+# ------------------------------------------------------------------------- dynamic-tanh stream, rotary attention with
+# head norms, mLSTM, group-limited routing
+def dyt_norm(x, alpha, w, b, rows=None, dtype=torch.float32):
+    """tanh(alpha x) * w + b of fp32 rows (``rows``: only these), in ``dtype``."""
+    xr = x if rows is None else x.index_select(0, rows)
+    return (torch.tanh(alpha * xr) * w + b).to(dtype)
+
+
+def residual_dyt_(x, y1, y2, bias, norm, out, assign=False):
+    """fp32 stream in place: ``x += y1 (+ y2) (+ bias)`` (the sub-layer outputs are summed first), or
+    ``x = y1`` when ``assign``; ``norm`` = (alpha, w, b): ``out`` takes tanh(alpha x) * w + b."""
+    if assign:
+        x.copy_(y1.float())
+    else:
+        y = y1.float()
+        if y2 is not None:
+            y = y + y2.float()
+        if bias is not None:
+            y = y + bias
+        x.add_(y)
+    if norm is not None:
+        out.copy_(torch.tanh(norm[0] * x) * norm[1] + norm[2])
+    return x
+
+
+def pack_pair(a, b, dtype):
+    """[a | b] rows of two fp32 streams, in ``dtype``."""
+    return torch.cat([a, b], dim=1).to(dtype)
+
+
+def bias_gelu_tanh_(x, bias):
+    """x = gelu_tanh(x + bias) in place (fp32 math; ``bias`` fp32 or None)."""
+    xf = x.float() if bias is None else x.float() + bias
+    x.copy_(torch.nn.functional.gelu(xf, approximate="tanh").to(x.dtype))
+    return x
+
+
+def rope_headnorm_cache_(proj, pos, slots, kc, vc, H, G, dk, dv, freq, mag, rot_dims, eps, q_w=None, k_w=None,
+                         v_off=None):
+    """See :func:`nv_genai_amd.ops.rope_headnorm_cache_`."""
+    T = proj.shape[0]
+    n0, n1 = H * dk, (H + G) * dk
+    q = proj[:, :n0].float().view(T, H, dk)
+    k = proj[:, n0:n1].float().view(T, G, dk)
+    v = k.clone() if v_off is None else proj[:, v_off:v_off + G * dv].float().view(T, G, dv)
+    if q_w is not None:
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_w
+    if k_w is not None:
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_w
+    cos, sin = rotary_cos_sin(pos.clamp(min=0), freq, mag)
+    q, k = _rotate(q, cos, sin, rot_dims, False), _rotate(k, cos, sin, rot_dims, False)
+    proj[:, :n0] = q.reshape(T, n0).to(proj.dtype)
+    proj[:, n0:n1] = k.reshape(T, n1 - n0).to(proj.dtype)
+    sl = slots.long()
+    ok = sl >= 0
+    BS = kc.shape[2]
+    blk, off = sl[ok] // BS, sl[ok] % BS
+    kc[blk, :, off, :] = k[ok].to(kc.dtype)
+    vc[blk, :, off, :] = v[ok].to(vc.dtype)
+    return proj
+
+
+def mlstm_scan(proj, gate_bias, state, H, d, dv, cap, cu, slots, pos, offs):
+    """See :func:`nv_genai_amd.ops.mlstm_scan`."""
+    T = proj.shape[0]
+    n = slots.numel()
+    qo, ko, vo, io = offs
+    pf = proj.float()
+    q = pf[:, qo:qo + H * d].reshape(T, H, d) * (d ** -0.5)
+    k = pf[:, ko:ko + H * d].reshape(T, H, d)
+    v = pf[:, vo:vo + H * dv].reshape(T, H, dv)
+    z = pf[:, io:io + 2 * H] + gate_bias
+    z = cap * torch.tanh(z / cap)
+    ig, fg = z[:, :H], torch.nn.functional.logsigmoid(z[:, H:])
+    out = torch.zeros(T, H, dv, dtype=torch.float32, device=proj.device)
+    for b in range(n):
+        t0, t1 = (b, b + 1) if cu is None else (int(cu[b]), int(cu[b + 1]))
+        if t1 <= t0:
+            continue
+        sl = int(slots[b])
+        if int(pos[t0]) == 0 or sl < 0:
+            S = torch.zeros(H, d, dv, dtype=torch.float32, device=proj.device)
+            nn = torch.zeros(H, d, dtype=torch.float32, device=proj.device)
+            m = torch.zeros(H, dtype=torch.float32, device=proj.device)
+        else:
+            st = state[sl]
+            S, nn, m = st[:, :d * dv].reshape(H, d, dv).clone(), st[:, d * dv:d * dv + d].clone(), st[:, d * dv + d].clone()
+        for t in range(t0, t1):
+            m_new = torch.maximum(fg[t] + m, ig[t])
+            a, bb = torch.exp(fg[t] + m - m_new), torch.exp(ig[t] - m_new)
+            S = a[:, None, None] * S + bb[:, None, None] * (k[t][:, :, None] * v[t][:, None, :])
+            nn = a[:, None] * nn + bb[:, None] * k[t]
+            m = m_new
+            den = torch.maximum((nn * q[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
+            out[t] = torch.einsum("hdv,hd->hv", S, q[t]) / den[:, None]
+        if sl >= 0:
+            state[sl] = torch.cat([S.reshape(H, d * dv), nn, m[:, None]], dim=1)
+    return out.reshape(T, H * dv)
+
+
+def moe_route_grouped(logits, correction, k, groups, keep, scale):
+    """See :func:`nv_genai_amd.ops.moe_route_grouped`."""
+    T, E = logits.shape
+    s = torch.softmax(logits.float(), -1)
+    c = s + correction
+    if groups > 1:
+        per = E // groups
+        best = c.view(T, groups, per).max(-1).values
+        _, gi = torch.sort(best, dim=-1, descending=True, stable=True)
+        kept = torch.zeros(T, groups, dtype=torch.bool, device=logits.device)
+        kept.scatter_(1, gi[:, :keep], True)
+        c = c.masked_fill(~kept.repeat_interleave(per, dim=1), float("-inf"))
+    _, ids = torch.sort(c, dim=-1, descending=True, stable=True)
+    ids = ids[:, :k]
+    w = torch.gather(s, 1, ids)
+    w = w / (w.sum(-1, keepdim=True) + 1e-20) * scale
+    return ids.to(torch.int32), w
