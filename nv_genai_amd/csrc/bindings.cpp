@@ -259,7 +259,7 @@ void moe_route_scores(Tensor logits, int64_t k, int64_t score, bool renorm, Tens
 // mode 0: out [M, F] = clamped_glu(s (A[sorted_tok] W_e[:F]^T), s (A[sorted_tok] W_e[F:]^T)), s = sorted_w or 1
 // mode 1: out [M, N] = (A W_e^T) * (sorted_w or 1)
 void moe_gemm_rows(Tensor A, Tensor W, Tensor sorted_tok, Tensor sorted_w, Tensor tiles, int64_t mt, Tensor out,
-                   int64_t mode, double limit, double alpha, bool use_weight) {
+                   int64_t mode, double limit, double alpha, bool use_weight, double shift) {
   const bool f32 = act_f32(A);
   CHECK_CONTIG(W); CHECK_CONTIG(out);
   TORCH_CHECK(W.is_cuda() && out.is_cuda() && W.scalar_type() == A.scalar_type() && out.scalar_type() == A.scalar_type());
@@ -291,10 +291,28 @@ void moe_gemm_rows(Tensor A, Tensor W, Tensor sorted_tok, Tensor sorted_w, Tenso
   p.limit = (float)limit;
   p.alpha = (float)alpha;
   p.use_weight = use_weight ? 1 : 0;
+  p.shift = (float)shift;
   nga::launch_moe_gemm_rows(p, (int)mode, f32, cur_stream(out));
 }
 
-void moe_combine_rows(Tensor y, Tensor inv, int64_t T, int64_t k, c10::optional<Tensor> add, Tensor out) {
+void moe_route_grouped(Tensor logits, Tensor correction, int64_t k, int64_t groups, int64_t keep, double scale,
+                       Tensor ids, Tensor w) {
+  CHECK_DEV(logits); CHECK_DT(logits, at::kFloat);
+  CHECK_DEV(correction); CHECK_DT(correction, at::kFloat); CHECK_CONTIG(correction);
+  TORCH_CHECK(logits.dim() == 2 && logits.stride(1) == 1, "moe_route_grouped: logits must be [T, E]");
+  const int64_t T = logits.size(0), E = logits.size(1);
+  TORCH_CHECK(correction.numel() == E && E >= 1 && E <= 512, "moe_route_grouped: one correction per expert, E <= 512");
+  TORCH_CHECK(groups >= 1 && groups <= 64 && E % groups == 0 && keep >= 1 && keep <= groups && k >= 1 &&
+              k <= keep * (E / groups), "moe_route_grouped: groups / keep / k do not fit the experts");
+  CHECK_DEV(ids); CHECK_DT(ids, at::kInt); CHECK_DEV(w); CHECK_DT(w, at::kFloat);
+  TORCH_CHECK(ids.is_contiguous() && w.is_contiguous() && ids.numel() >= T * k && w.numel() >= T * k);
+  nga::launch_moe_route_grouped(logits.data_ptr<float>(), logits.stride(0), correction.data_ptr<float>(), (int)T, (int)E,
+                                (int)k, (int)groups, (int)keep, (float)scale, ids.data_ptr<int32_t>(),
+                                w.data_ptr<float>(), cur_stream(logits));
+}
+
+void moe_combine_rows(Tensor y, Tensor inv, int64_t T, int64_t k, c10::optional<Tensor> add, Tensor out,
+                      c10::optional<Tensor> id_x, c10::optional<Tensor> ids, c10::optional<Tensor> wts, int64_t E) {
   const bool f32 = act_f32(y);
   CHECK_CONTIG(y); CHECK_CONTIG(out);
   CHECK_DEV(inv); CHECK_DT(inv, at::kInt);
@@ -309,8 +327,24 @@ void moe_combine_rows(Tensor y, Tensor inv, int64_t T, int64_t k, c10::optional<
     ap = add->data_ptr();
     as = add->stride(0);
   }
+  const void* xp = nullptr;
+  int64_t xs = 0;
+  const int32_t* idp = nullptr;
+  const float* wp = nullptr;
+  if (id_x.has_value()) {   // identity experts: ids >= E add weight * the token's own row
+    TORCH_CHECK(ids.has_value() && wts.has_value(), "identity experts need the ids and weights");
+    TORCH_CHECK(id_x->is_cuda() && id_x->scalar_type() == y.scalar_type() && id_x->dim() == 2 && id_x->size(0) == T &&
+                id_x->size(1) == out.size(1) && id_x->stride(1) == 1, "id_x must be [T, H] rows");
+    CHECK_DEV(*ids); CHECK_DT(*ids, at::kInt); CHECK_CONTIG(*ids);
+    CHECK_DEV(*wts); CHECK_DT(*wts, at::kFloat); CHECK_CONTIG(*wts);
+    TORCH_CHECK(ids->numel() >= T * k && wts->numel() >= T * k);
+    xp = id_x->data_ptr();
+    xs = id_x->stride(0);
+    idp = ids->data_ptr<int32_t>();
+    wp = wts->data_ptr<float>();
+  }
   nga::launch_moe_combine_rows(y.data_ptr(), inv.data_ptr<int32_t>(), (int)T, (int)k, (int)out.size(1), ap, as,
-                               out.data_ptr(), f32, cur_stream(y));
+                               out.data_ptr(), xp, xs, idp, wp, (int)E, f32, cur_stream(y));
 }
 
 void moe_combine(Tensor y, Tensor inv, int64_t T, int64_t k, Tensor out) {
@@ -1265,14 +1299,14 @@ void residual_add_rmsnorm(Tensor x, Tensor y, c10::optional<Tensor> w, double ep
                                    (float)eps, x.size(0), (int)H, op, f32, cur_stream(x));
 }
 
-void clamped_glu(Tensor out, Tensor x, int64_t F, double limit, double alpha, int64_t gate_col) {
+void clamped_glu(Tensor out, Tensor x, int64_t F, double limit, double alpha, int64_t gate_col, double shift) {
   const bool f32 = act_f32(x);
   CHECK_CONTIG(out);
   TORCH_CHECK(out.is_cuda() && out.scalar_type() == x.scalar_type());
   TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1 && F >= 1 && x.size(1) >= 2 * F && gate_col < x.size(1));
   TORCH_CHECK(out.dim() == 2 && out.size(0) == x.size(0) && out.size(1) == F);
   nga::launch_clamped_glu(out.data_ptr(), x.data_ptr(), x.stride(0), x.size(0), (int)F, (float)limit, (float)alpha,
-                          (int)gate_col, f32, cur_stream(x));
+                          (int)gate_col, (float)shift, f32, cur_stream(x));
 }
 
 void latent_rope_cache(Tensor proj, Tensor pos, Tensor slots, c10::optional<Tensor> page, Tensor freq, double mag,
@@ -1333,13 +1367,153 @@ void latent_rope_cache(Tensor proj, Tensor pos, Tensor slots, c10::optional<Tens
   nga::launch_latent_rope_cache(p, T, f32, cur_stream(proj));
 }
 
-void group_rmsnorm(Tensor out, Tensor x, Tensor w, int64_t groups, double eps) {
+void group_rmsnorm(Tensor out, Tensor x, Tensor w, int64_t groups, double eps, c10::optional<Tensor> gate) {
   CHECK_F32(x); CHECK_F32(w); CHECK_CONTIG(out);
   const bool f32 = act_f32(out);
   TORCH_CHECK(x.dim() == 2 && out.sizes() == x.sizes() && groups > 0 && x.size(1) % groups == 0 &&
-              w.numel() == x.size(1) / groups);
-  nga::launch_group_rmsnorm(out.data_ptr(), x.data_ptr<float>(), w.data_ptr<float>(), x.size(0), (int)groups,
+              (w.numel() == x.size(1) / groups || w.numel() == x.size(1)));
+  const void* gp = nullptr;
+  int64_t gs = 0;
+  if (gate.has_value()) {
+    TORCH_CHECK(gate->is_cuda() && gate->scalar_type() == out.scalar_type() && gate->dim() == 2 &&
+                gate->size(0) == x.size(0) && gate->size(1) == x.size(1) && gate->stride(1) == 1,
+                "gate: [T, columns] rows of the output type");
+    gp = gate->data_ptr();
+    gs = gate->stride(0);
+  }
+  nga::launch_group_rmsnorm(out.data_ptr(), x.data_ptr<float>(), w.data_ptr<float>(),
+                            groups > 1 && w.numel() == x.size(1), gp, gs, x.size(0), (int)groups,
                             (int)(x.size(1) / groups), (float)eps, f32, cur_stream(x));
+}
+
+// ------------------------------------------------------------------ dynamic-tanh stream, rotary attention with head norms
+void dyt_norm(Tensor out, Tensor x, double alpha, Tensor w, Tensor b, c10::optional<Tensor> rows) {
+  CHECK_F32(x); CHECK_F32(w); CHECK_F32(b); CHECK_CONTIG(out);
+  const bool f32 = act_f32(out);
+  const int64_t H = x.size(1);
+  TORCH_CHECK(x.dim() == 2 && out.dim() == 2 && out.size(1) == H && w.numel() == H && b.numel() == H);
+  const int64_t* rp = nullptr;
+  if (rows.has_value()) {
+    CHECK_DEV(*rows); CHECK_DT(*rows, at::kLong); CHECK_CONTIG(*rows);
+    TORCH_CHECK(rows->numel() == out.size(0));
+    rp = rows->data_ptr<int64_t>();
+  } else {
+    TORCH_CHECK(out.size(0) == x.size(0));
+  }
+  nga::launch_dyt_norm(out.data_ptr(), x.data_ptr<float>(), (float)alpha, w.data_ptr<float>(), b.data_ptr<float>(), rp,
+                       out.size(0), (int)H, f32, cur_stream(x));
+}
+
+void residual_dyt(Tensor x, Tensor y1, c10::optional<Tensor> y2, c10::optional<Tensor> bias, double alpha,
+                  c10::optional<Tensor> w, c10::optional<Tensor> b, c10::optional<Tensor> out, bool assign) {
+  CHECK_F32(x);
+  const bool f32 = act_f32(y1);
+  const int64_t T = x.size(0), H = x.size(1);
+  TORCH_CHECK(x.dim() == 2 && y1.dim() == 2 && y1.size(0) == T && y1.size(1) == H && y1.stride(1) == 1);
+  const void* y2p = nullptr;
+  int64_t s2 = 0;
+  if (y2.has_value()) {
+    TORCH_CHECK(!assign, "residual_dyt: one source replaces the stream");
+    TORCH_CHECK(y2->is_cuda() && y2->scalar_type() == y1.scalar_type() && y2->dim() == 2 && y2->size(0) == T &&
+                y2->size(1) == H && y2->stride(1) == 1);
+    y2p = y2->data_ptr();
+    s2 = y2->stride(0);
+  }
+  TORCH_CHECK(out.has_value() == w.has_value() && out.has_value() == b.has_value(),
+              "residual_dyt: weight, bias and output of the norm come together");
+  void* op = nullptr;
+  if (out.has_value()) {
+    CHECK_CONTIG(*out);
+    TORCH_CHECK(out->is_cuda() && out->scalar_type() == y1.scalar_type() && out->sizes() == x.sizes());
+    op = out->data_ptr();
+  }
+  nga::launch_residual_dyt(x.data_ptr<float>(), y1.data_ptr(), y1.stride(0), y2p, s2, opt_f32(bias, H, "bias row"),
+                           (float)alpha, opt_f32(w, H, "norm weight"), opt_f32(b, H, "norm bias"), op, T, (int)H, assign,
+                           f32, cur_stream(x));
+}
+
+void pack_pair(Tensor out, Tensor a, Tensor b) {
+  CHECK_F32(a); CHECK_F32(b); CHECK_CONTIG(out);
+  const bool f32 = act_f32(out);
+  TORCH_CHECK(a.dim() == 2 && b.dim() == 2 && a.size(0) == b.size(0) && out.dim() == 2 && out.size(0) == a.size(0) &&
+              out.size(1) == a.size(1) + b.size(1));
+  nga::launch_pack_pair(out.data_ptr(), a.data_ptr<float>(), b.data_ptr<float>(), a.size(0), (int)a.size(1),
+                        (int)b.size(1), f32, cur_stream(a));
+}
+
+void bias_gelu_tanh(Tensor x, c10::optional<Tensor> bias) {
+  const bool f32 = act_f32(x);
+  CHECK_CONTIG(x);
+  TORCH_CHECK(x.dim() == 2);
+  nga::launch_bias_gelu_tanh(x.data_ptr(), opt_f32(bias, x.size(1), "bias"), x.size(0), (int)x.size(1), f32,
+                             cur_stream(x));
+}
+
+void rope_headnorm_cache(Tensor proj, Tensor pos, Tensor slots, Tensor kc, Tensor vc, int64_t H, int64_t G, int64_t dk,
+                         int64_t dv, Tensor freq, double mag, int64_t rot_dims, double eps, c10::optional<Tensor> q_w,
+                         c10::optional<Tensor> k_w, int64_t v_off) {
+  const bool f32 = act_f32(proj);
+  CHECK_I32(pos); CHECK_I32(slots);
+  const int64_t T = proj.size(0), W = proj.size(1);
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && pos.numel() == T && slots.numel() == T);
+  TORCH_CHECK(H >= 1 && G >= 1 && dk >= 1 && dk <= 512 && dv >= 1 && (H + G) * dk <= W, "q / k heads outside the rows");
+  TORCH_CHECK(freq.is_cuda() && freq.scalar_type() == at::kDouble && freq.is_contiguous(), "freq: float64 on the GPU");
+  TORCH_CHECK(rot_dims >= 2 && rot_dims % 2 == 0 && rot_dims <= dk && freq.numel() == rot_dims / 2,
+              "rotary positions: an even number of elements <= dk");
+  TORCH_CHECK(v_off < 0 ? dv == dk : (v_off >= (H + G) * dk && v_off + G * dv <= W), "value columns outside the rows");
+  check_row_pages(proj, kc, G, dk, "rope_headnorm_cache");
+  check_row_pages(proj, vc, G, dv, "rope_headnorm_cache");
+  TORCH_CHECK(kc.size(0) == vc.size(0));
+  nga::RopeHeadnormParams p{};
+  p.proj = proj.data_ptr();
+  p.stride = proj.stride(0);
+  p.pos = pos.data_ptr<int32_t>();
+  p.slots = slots.data_ptr<int32_t>();
+  p.kc = kc.data_ptr();
+  p.vc = vc.data_ptr();
+  p.freq = freq.data_ptr<double>();
+  p.mag = (float)mag;
+  p.eps = (float)eps;
+  p.H = (int)H;
+  p.G = (int)G;
+  p.dk = (int)dk;
+  p.dv = (int)dv;
+  p.rot_dims = (int)rot_dims;
+  p.q_w = opt_f32(q_w, dk, "q head norm weight");
+  p.k_w = opt_f32(k_w, dk, "k head norm weight");
+  p.v_off = (int)v_off;
+  nga::launch_rope_headnorm_cache(p, T, f32, cur_stream(proj));
+}
+
+void mlstm_scan(Tensor out, Tensor proj, Tensor gate_bias, Tensor state, int64_t H, int64_t d, int64_t dv, double cap,
+                c10::optional<Tensor> cu, Tensor slots, Tensor pos, int64_t q_off, int64_t k_off, int64_t v_off,
+                int64_t g_off) {
+  const bool f32 = act_f32(proj);
+  CHECK_F32(out); CHECK_F32(gate_bias); CHECK_F32(state); CHECK_I32(slots); CHECK_I32(pos);
+  CHECK_CONTIG(out); CHECK_CONTIG(state);
+  const int64_t T = proj.size(0), W = proj.size(1);
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && H >= 1 && d >= 1 && dv >= 1 && cap > 0);
+  TORCH_CHECK(q_off >= 0 && k_off >= 0 && v_off >= 0 && g_off >= 0 && q_off + H * d <= W && k_off + H * d <= W &&
+              v_off + H * dv <= W && g_off + 2 * H <= W, "mlstm_scan: columns outside the rows");
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == H * dv && pos.numel() == T);
+  TORCH_CHECK(gate_bias.numel() == 2 * H);
+  TORCH_CHECK(state.dim() == 3 && state.size(1) == H && state.size(2) == d * dv + d + 1,
+              "mlstm_scan: state must be [slots, H, d * dv + d + 1]");
+  TORCH_CHECK(d <= nga::mlstm_max_dim(), "mlstm_scan: the per-head key size exceeds the kernel's register tile");
+  const int n = (int)slots.numel();
+  const int32_t* cp = nullptr;
+  if (cu.has_value()) {
+    CHECK_I32(*cu);
+    TORCH_CHECK(cu->numel() == n + 1);
+    cp = cu->data_ptr<int32_t>();
+  } else {
+    TORCH_CHECK(n == T, "mlstm_scan: without cu every row is a segment");
+  }
+  TORCH_CHECK(nga::launch_mlstm_scan(out.data_ptr<float>(), proj.data_ptr(), proj.stride(0), gate_bias.data_ptr<float>(),
+                                     state.data_ptr<float>(), (int)H, (int)d, (int)dv, (float)cap, cp,
+                                     slots.data_ptr<int32_t>(), pos.data_ptr<int32_t>(), n, (int)q_off, (int)k_off,
+                                     (int)v_off, (int)g_off, f32, cur_stream(proj)),
+              "mlstm_scan: no kernel for these sizes");
 }
 
 // K [blocks, nk, 64, dk] and V [blocks, nv, 64, dv] pages of the activation type
@@ -1422,7 +1596,8 @@ SoftmaxArgs check_softmax_args(const Tensor& out, const Tensor& q, const c10::op
 
 void softmax_attention(Tensor out, Tensor q, c10::optional<Tensor> gate, Tensor kc, Tensor vc, Tensor block_tables,
                        Tensor tok_seq, Tensor pos, int64_t H, int64_t G, int64_t dk, int64_t dv, double scale,
-                       int64_t window, int64_t maps, double lam, double unit_eps, double out_scale, bool v_in_k) {
+                       int64_t window, int64_t maps, double lam, double unit_eps, double out_scale, bool v_in_k,
+                       double softcap) {
   const bool f32 = act_f32(q);
   CHECK_I32(block_tables); CHECK_I32(tok_seq); CHECK_I32(pos);
   const SoftmaxArgs a = check_softmax_args(out, q, gate, kc, vc, H, G, dk, dv, window, maps, v_in_k);
@@ -1432,7 +1607,7 @@ void softmax_attention(Tensor out, Tensor q, c10::optional<Tensor> gate, Tensor 
                                 block_tables.data_ptr<int32_t>(), (int)block_tables.size(1),
                                 tok_seq.data_ptr<int32_t>(), pos.data_ptr<int32_t>(), T, (int)H, (int)G, (int)dk,
                                 (int)dv, (float)scale, (int)window, (int)maps, (float)lam, (float)unit_eps,
-                                (float)out_scale, v_in_k, f32, cur_stream(q));
+                                (float)out_scale, v_in_k, (float)softcap, f32, cur_stream(q));
 }
 
 // prompt portions on the MFMA kernel (bf16): sequence b owns rows [cu_q[b], cu_q[b + 1]) of q / gate / out,
@@ -1440,7 +1615,7 @@ void softmax_attention(Tensor out, Tensor q, c10::optional<Tensor> gate, Tensor 
 void softmax_attention_prefill(Tensor out, Tensor q, c10::optional<Tensor> gate, Tensor kc, Tensor vc,
                                Tensor block_tables, Tensor cu_q, Tensor ctx_lens, int64_t max_q_len, int64_t H,
                                int64_t G, int64_t dk, int64_t dv, double scale, int64_t window, int64_t maps, double lam,
-                               double unit_eps, double out_scale, bool v_in_k) {
+                               double unit_eps, double out_scale, bool v_in_k, double softcap) {
   CHECK_BF16(q); CHECK_BF16(out); CHECK_I32(block_tables); CHECK_I32(cu_q); CHECK_I32(ctx_lens);
   const SoftmaxArgs a = check_softmax_args(out, q, gate, kc, vc, H, G, dk, dv, window, maps, v_in_k);
   TORCH_CHECK(nga::softmax_attention_mfma_supported((int)dk, (int)dv, (int)(H / G), (int)maps),
@@ -1452,14 +1627,14 @@ void softmax_attention_prefill(Tensor out, Tensor q, c10::optional<Tensor> gate,
                                      block_tables.data_ptr<int32_t>(), (int)block_tables.size(1),
                                      cu_q.data_ptr<int32_t>(), ctx_lens.data_ptr<int32_t>(), (int)B, (int)max_q_len,
                                      (int)H, (int)G, (int)dk, (int)dv, (float)scale, (int)window, (int)maps, (float)lam,
-                                     (float)unit_eps, (float)out_scale, v_in_k, cur_stream(q));
+                                     (float)unit_eps, (float)out_scale, v_in_k, (float)softcap, cur_stream(q));
 }
 
 // single-token rows on the MFMA kernel (bf16): ws is the fp32 partial workspace [T, H, maps, parts, dv + 4]
 void softmax_attention_decode(Tensor out, Tensor ws, int64_t parts, Tensor q, c10::optional<Tensor> gate, Tensor kc,
                               Tensor vc, Tensor block_tables, Tensor tok_seq, Tensor pos, int64_t H, int64_t G,
                               int64_t dk, int64_t dv, double scale, int64_t window, int64_t maps, double lam,
-                              double unit_eps, double out_scale, bool v_in_k) {
+                              double unit_eps, double out_scale, bool v_in_k, double softcap) {
   CHECK_BF16(q); CHECK_BF16(out); CHECK_F32(ws); CHECK_I32(block_tables); CHECK_I32(tok_seq); CHECK_I32(pos);
   const SoftmaxArgs a = check_softmax_args(out, q, gate, kc, vc, H, G, dk, dv, window, maps, v_in_k);
   TORCH_CHECK(nga::softmax_attention_mfma_supported((int)dk, (int)dv, (int)(H / G), (int)maps),
@@ -1473,7 +1648,7 @@ void softmax_attention_decode(Tensor out, Tensor ws, int64_t parts, Tensor q, c1
                                   (const uint16_t*)a.gp, a.gs, bfp(kc), bfp(vc), block_tables.data_ptr<int32_t>(),
                                   (int)block_tables.size(1), tok_seq.data_ptr<int32_t>(), pos.data_ptr<int32_t>(), T,
                                   (int)H, (int)G, (int)dk, (int)dv, (float)scale, (int)window, (int)maps, (float)lam,
-                                  (float)unit_eps, (float)out_scale, v_in_k, cur_stream(q));
+                                  (float)unit_eps, (float)out_scale, v_in_k, (float)softcap, cur_stream(q));
 }
 
 void hgrn2_scan(Tensor out, Tensor proj, Tensor f_bias, Tensor lower, Tensor state, int64_t H, int64_t d, int64_t dv,
@@ -1566,6 +1741,13 @@ PYBIND11_MODULE(_C, m) {
   m.def("headnorm_cache", checked("headnorm_cache", &headnorm_cache));
   m.def("softmax_attention", checked("softmax_attention", &softmax_attention));
   m.def("hgrn2_scan", checked("hgrn2_scan", &hgrn2_scan));
+  m.def("mlstm_scan", checked("mlstm_scan", &mlstm_scan));
+  m.def("dyt_norm", checked("dyt_norm", &dyt_norm));
+  m.def("residual_dyt", checked("residual_dyt", &residual_dyt));
+  m.def("pack_pair", checked("pack_pair", &pack_pair));
+  m.def("bias_gelu_tanh", checked("bias_gelu_tanh", &bias_gelu_tanh));
+  m.def("rope_headnorm_cache", checked("rope_headnorm_cache", &rope_headnorm_cache));
+  m.def("moe_route_grouped", checked("moe_route_grouped", &moe_route_grouped));
   m.def("softmax_attention_mfma_supported", [](int64_t dk, int64_t dv, int64_t group, int64_t maps) {
     return nga::softmax_attention_mfma_supported((int)dk, (int)dv, (int)group, (int)maps);
   });

@@ -185,12 +185,17 @@ struct MoeRowsParams {
   int64_t ldo;
   float limit, alpha;
   int use_weight;            // scale by the routing weight (MODE 0: gate and up before the activation)
+  float shift;               // MODE 0 epilogue: g sigmoid(alpha g) (u + shift)
 };
 void launch_moe_route_scores(const float* logits, int64_t ld, int T, int E, int k, int score, bool renorm,
                              int32_t* ids, float* w, hipStream_t stream);
 void launch_moe_gemm_rows(const MoeRowsParams& p, int mode, bool f32, hipStream_t stream);
+// id_x != nullptr: assignments with ids >= E are identity experts, out += w * id_x row
 void launch_moe_combine_rows(const void* y, const int32_t* inv, int T, int k, int H, const void* add,
-                             int64_t add_stride, void* out, bool f32, hipStream_t stream);
+                             int64_t add_stride, void* out, const void* id_x, int64_t id_stride, const int32_t* ids,
+                             const float* wts, int E, bool f32, hipStream_t stream);
+void launch_moe_route_grouped(const float* logits, int64_t ld, const float* correction, int T, int E, int k, int groups,
+                              int keep, float scale, int32_t* ids, float* w, hipStream_t stream);
 void launch_moe_route(const uint16_t* logits, int64_t ld, int T, int E, int k, int32_t* ids,
                       float* w, hipStream_t stream);
 void launch_moe_align(const int32_t* ids, const float* w, int M, int k, int e0, int E, int bm,
@@ -294,7 +299,14 @@ void launch_softcap(float* z, int64_t n, float cap, float scale, hipStream_t str
 void launch_residual_add_rmsnorm(float* x, const void* y, int64_t y_stride, const float* w, float eps, int64_t T, int H,
                                  void* out, bool f32, hipStream_t stream);
 void launch_clamped_glu(void* out, const void* in, int64_t in_stride, int64_t T, int F, float limit, float alpha,
-                        int gate_col, bool f32, hipStream_t stream);
+                        int gate_col, float shift, bool f32, hipStream_t stream);
+void launch_dyt_norm(void* out, const float* x, float alpha, const float* w, const float* b, const int64_t* rows,
+                     int64_t n_out, int H, bool f32, hipStream_t stream);
+void launch_residual_dyt(float* x, const void* y1, int64_t s1, const void* y2, int64_t s2, const float* bias, float alpha,
+                         const float* w, const float* b, void* out, int64_t T, int H, bool assign, bool f32,
+                         hipStream_t stream);
+void launch_pack_pair(void* out, const float* a, const float* b, int64_t T, int Ha, int Hb, bool f32, hipStream_t stream);
+void launch_bias_gelu_tanh(void* x, const float* bias, int64_t T, int F, bool f32, hipStream_t stream);
 
 // latent_rope.hip: latent norm + rotary positions + page write of latent attention with a rotated key part
 struct LatentRopeParams {
@@ -316,8 +328,25 @@ struct LatentRopeParams {
   const float* n_w;
 };
 void launch_latent_rope_cache(const LatentRopeParams& p, int64_t T, bool f32, hipStream_t stream);
-void launch_group_rmsnorm(void* out, const float* x, const float* w, int64_t T, int groups, int gs, float eps, bool f32,
-                          hipStream_t stream);
+// rope_headnorm_cache: rows [q: H heads of dk | k: G heads of dk | ...], head norms, rotary pairs (i, i + rot_dims / 2)
+struct RopeHeadnormParams {
+  void* proj;                // [T, stride] projection rows (activation type)
+  int64_t stride;
+  const int32_t* pos;        // [T]
+  const int32_t* slots;      // [T] page slot of the token (< 0: no write)
+  void* kc;                  // [blocks, G, 64, dk]
+  void* vc;                  // [blocks, G, 64, dv]
+  const double* freq;        // [rot_dims / 2]
+  float mag, eps;
+  int H, G, dk, dv, rot_dims;
+  const float* q_w;          // [dk] or nullptr: no norm of the q heads
+  const float* k_w;          // [dk] or nullptr
+  int v_off;                 // value columns [v_off, v_off + G * dv), or < 0: the k heads before norm and rotation
+};
+void launch_rope_headnorm_cache(const RopeHeadnormParams& p, int64_t T, bool f32, hipStream_t stream);
+// w: gs weights shared by the groups, or groups * gs (w_full); gate [T, groups * gs] rows of the output type or nullptr
+void launch_group_rmsnorm(void* out, const float* x, const float* w, bool w_full, const void* gate, int64_t g_stride,
+                          int64_t T, int groups, int gs, float eps, bool f32, hipStream_t stream);
 
 // softmax_attention.hip: K [blocks, G * maps, 64, dk], V [blocks, G, 64, dv] pages, bf16 or fp32
 void launch_headnorm_cache(void* proj, int64_t stride, const int32_t* slots, void* kc, void* vc, int64_t T, int nq,
@@ -327,7 +356,7 @@ void launch_softmax_attention(void* out, const void* q, int64_t q_stride, const 
                               const void* kc, const void* vc, const int32_t* block_tables, int max_blocks,
                               const int32_t* tok_seq, const int32_t* pos, int64_t T, int H, int G, int dk, int dv,
                               float scale, int window, int maps, float lam, float unit_eps, float out_scale, bool v_in_k,
-                              bool f32, hipStream_t stream);
+                              float softcap, bool f32, hipStream_t stream);
 
 bool softmax_attention_mfma_supported(int dk, int dv, int group, int maps);
 void launch_softmax_attention_mfma(uint16_t* out, const uint16_t* q, int64_t q_stride, const uint16_t* gate,
@@ -335,16 +364,21 @@ void launch_softmax_attention_mfma(uint16_t* out, const uint16_t* q, int64_t q_s
                                    const int32_t* block_tables, int max_blocks, const int32_t* cu_q,
                                    const int32_t* ctx_lens, int B, int max_q_len, int H, int G, int dk, int dv,
                                    float scale, int window, int maps, float lam, float unit_eps, float out_scale,
-                                   bool v_in_k, hipStream_t stream);
+                                   bool v_in_k, float softcap, hipStream_t stream);
 int softmax_decode_parts(int rows, int G, int max_ctx, int window);
 void launch_softmax_decode_mfma(uint16_t* out, float* ws, int parts, const uint16_t* q, int64_t q_stride,
                                 const uint16_t* gate, int64_t g_stride, const uint16_t* kc, const uint16_t* vc,
                                 const int32_t* block_tables, int max_blocks, const int32_t* tok_seq,
                                 const int32_t* pos, int64_t T, int H, int G, int dk, int dv, float scale, int window,
-                                int maps, float lam, float unit_eps, float out_scale, bool v_in_k,
+                                int maps, float lam, float unit_eps, float out_scale, bool v_in_k, float softcap,
                                 hipStream_t stream);
 
 // recurrent.hip
+int mlstm_max_dim();
+// state [slots, H, d * dv + d + 1] fp32 (S, n, m); gate columns [i (H) | f (H)] from g_off
+bool launch_mlstm_scan(float* out, const void* proj, int64_t stride, const float* gate_bias, float* state, int H, int d,
+                       int dv, float cap, const int32_t* cu, const int32_t* slots, const int32_t* pos, int n_seg,
+                       int q_off, int k_off, int v_off, int g_off, bool f32, hipStream_t stream);
 int hgrn2_max_dim(int dv);
 bool launch_hgrn2_scan(float* out, const void* proj, int64_t stride, const float* f_bias, const float* lower,
                        float* state, int H, int d, int dv, const int32_t* cu, const int32_t* slots, const int32_t* pos,

@@ -21,7 +21,9 @@
 //                operands, any K / F / N (experts too small or too odd for the MFMA tiles,
 //                and the true-fp32 path)
 //   moe_combine_rows  moe_combine for any width and type, plus an optional added row (a shared
-//                expert's output)
+//                expert's output) and identity experts (ids >= E: weight * the token's own row)
+//   moe_route_grouped fp32 router logits -> softmax scores, choice by score + correction inside
+//                the best groups of experts, top-k ids + weights renormalised and scaled
 //
 // GEMM: see the block comment above moe_gemm_kernel. Weight rows are the MFMA A operand and
 // token rows the B operand, so each lane
@@ -49,11 +51,11 @@ __device__ __forceinline__ float gelu_tanh(float x) {
   const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
   return x - x / (1.f + __expf(2.f * u));
 }
-// g sigmoid(alpha g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit)
-__device__ __forceinline__ float clamped_glu(float gate, float up, float limit, float alpha) {
+// g sigmoid(alpha g) (u + shift) with g = min(gate, limit), u = clamp(up, -limit, limit)
+__device__ __forceinline__ float clamped_glu(float gate, float up, float limit, float alpha, float shift = 1.f) {
   const float g = fminf(gate, limit);
   const float u = fminf(fmaxf(up, -limit), limit);
-  return g / (1.f + expf(-alpha * g)) * (u + 1.f);
+  return g / (1.f + expf(-alpha * g)) * (u + shift);
 }
 }  // namespace
 
@@ -329,10 +331,13 @@ __global__ void __launch_bounds__(256) moe_gemm_kernel(MoeGemmParams P) {
 }
 
 // ------------------------------------------------------------------ combine
-// out[t, :] = sum_j y[inv[t*k + j], :] (+ add[t, :]) (fp32), 8 features per thread
+// out[t, :] = sum_j y[inv[t*k + j], :] (+ add[t, :]) (+ identity experts' weight * x[t, :]) (fp32), 8 features per thread
 __global__ void moe_combine_kernel(const uint16_t* __restrict__ y, const int32_t* __restrict__ inv,
                                    int T, int k, int H, uint16_t* __restrict__ out,
-                                   const uint16_t* __restrict__ add = nullptr, int64_t add_stride = 0) {
+                                   const uint16_t* __restrict__ add = nullptr, int64_t add_stride = 0,
+                                   const uint16_t* __restrict__ id_x = nullptr, int64_t id_stride = 0,
+                                   const int32_t* __restrict__ ids = nullptr, const float* __restrict__ wts = nullptr,
+                                   int E = 0) {
   const int64_t vec = H / 8;
   const int64_t total = (int64_t)T * vec;
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
@@ -345,12 +350,21 @@ __global__ void moe_combine_kernel(const uint16_t* __restrict__ y, const int32_t
 #pragma unroll
       for (int q = 0; q < 8; ++q) a[q] = bf2f(v[q]);
     }
+    float idw = 0.f;   // weight of the row's identity experts (ids >= E): they return the row itself
     for (int j = 0; j < k; ++j) {
       const int p = inv[t * k + j];
-      if (p < 0) continue;
+      if (p < 0) {
+        if (id_x && ids[t * k + j] >= E) idw += wts[t * k + j];
+        continue;
+      }
       const u16x8 v = load8(y + (int64_t)p * H + c);
 #pragma unroll
       for (int q = 0; q < 8; ++q) a[q] += bf2f(v[q]);
+    }
+    if (idw != 0.f) {
+      const u16x8 v = load8(id_x + t * id_stride + c);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) a[q] += idw * bf2f(v[q]);
     }
     u16x8 o;
 #pragma unroll
@@ -401,6 +415,82 @@ __global__ void moe_route_scores_kernel(const float* __restrict__ logits, int64_
     ids[(int64_t)t * k + j] = sel[j];
     w[(int64_t)t * k + j] = renorm ? top[j] / sum : top[j];
   }
+}
+
+
+// ------------------------------------------------------------------ group-limited routing
+// One thread per token. Scores s = softmax(logits) over all E (fp32); the choice is made by
+// c = s + correction among the `keep` groups (of E / groups neighbouring experts) whose largest c
+// is largest; the k largest c inside the kept groups (ties: the lower index) get the weights
+// s / (sum of the chosen s + 1e-20) * scale. Scores live in the workgroup's LDS, one column per
+// thread, so E is bounded only by LDS (E <= 512 at 32 threads).
+constexpr int RG_THREADS = 32, RG_MAX_E = 512, RG_MAX_GROUPS = 64;
+__global__ void __launch_bounds__(RG_THREADS) moe_route_grouped_kernel(
+    const float* __restrict__ logits, int64_t ld, const float* __restrict__ correction, int T, int E, int k, int groups,
+    int keep, float scale, int32_t* __restrict__ ids, float* __restrict__ w) {
+  extern __shared__ float rg_s[];   // [E][RG_THREADS] scores, then [E][RG_THREADS] choice scores
+  const int t = blockIdx.x * RG_THREADS + threadIdx.x;
+  if (t >= T) return;
+  float* s = rg_s + threadIdx.x;
+  float* c = rg_s + (int64_t)E * RG_THREADS + threadIdx.x;
+  const float* lp = logits + (int64_t)t * ld;
+  float mx = -INFINITY;
+  for (int e = 0; e < E; ++e) mx = fmaxf(mx, lp[e]);
+  float den = 0.f;
+  for (int e = 0; e < E; ++e) {
+    const float v = expf(lp[e] - mx);
+    s[e * RG_THREADS] = v;
+    den += v;
+  }
+  for (int e = 0; e < E; ++e) {
+    const float v = s[e * RG_THREADS] / den;
+    s[e * RG_THREADS] = v;
+    c[e * RG_THREADS] = v + correction[e];
+  }
+  if (groups > 1) {
+    const int per = E / groups;
+    uint64_t kept = 0;
+    for (int j = 0; j < keep; ++j) {
+      float best = 0.f;
+      int bg = -1;
+      for (int g = 0; g < groups; ++g) {
+        if ((kept >> g) & 1ull) continue;
+        float gm = -INFINITY;
+        for (int e = g * per; e < (g + 1) * per; ++e) gm = fmaxf(gm, c[e * RG_THREADS]);
+        if (bg < 0 || gm > best) {
+          best = gm;
+          bg = g;
+        }
+      }
+      kept |= 1ull << bg;
+    }
+    for (int g = 0; g < groups; ++g)
+      if (!((kept >> g) & 1ull))
+        for (int e = g * per; e < (g + 1) * per; ++e) c[e * RG_THREADS] = -INFINITY;
+  }
+  float sum = 0.f;
+  for (int j = 0; j < k; ++j) {
+    float best = 0.f;
+    int bi = -1;
+    for (int e = 0; e < E; ++e) {
+      const float v = c[e * RG_THREADS];
+      if (v == -INFINITY && bi >= 0) continue;
+      if (bi < 0 || v > best) {
+        bool taken = false;
+        for (int i = 0; i < j; ++i) taken |= ids[(int64_t)t * k + i] == e;
+        if (!taken) {
+          best = v;
+          bi = e;
+        }
+      }
+    }
+    ids[(int64_t)t * k + j] = bi;
+    const float sv = s[bi * RG_THREADS];
+    w[(int64_t)t * k + j] = sv;
+    sum += sv;
+  }
+  const float r = scale / (sum + 1e-20f);
+  for (int j = 0; j < k; ++j) w[(int64_t)t * k + j] *= r;
 }
 
 // ------------------------------------------------------------------ grouped GEMM on VALU tiles
@@ -489,7 +579,7 @@ __global__ void __launch_bounds__(256) moe_gemm_rows_kernel(MoeRowsParams P) {
     for (int j = 0; j < 4; ++j) {
       const int n = nb * RT + 4 * tc + j;
       if (n >= N) continue;
-      const float v = MODE == 0 ? clamped_glu(accA[i][j] * sw, accB[i][j] * sw, P.limit, P.alpha) : accA[i][j] * sw;
+      const float v = MODE == 0 ? clamped_glu(accA[i][j] * sw, accB[i][j] * sw, P.limit, P.alpha, P.shift) : accA[i][j] * sw;
       stv(out + (int64_t)pos * P.ldo + n, v);
     }
   }
@@ -499,14 +589,22 @@ __global__ void __launch_bounds__(256) moe_gemm_rows_kernel(MoeRowsParams P) {
 template <typename T>
 __global__ void __launch_bounds__(256) moe_combine_rows_kernel(const T* __restrict__ y, const int32_t* __restrict__ inv,
                                                                int k, int H, const T* __restrict__ add,
-                                                               int64_t add_stride, T* __restrict__ out) {
+                                                               int64_t add_stride, T* __restrict__ out,
+                                                               const T* __restrict__ id_x, int64_t id_stride,
+                                                               const int32_t* __restrict__ ids,
+                                                               const float* __restrict__ wts, int E) {
   const int64_t t = blockIdx.x;
+  float idw = 0.f;   // weight of the row's identity experts (ids >= E)
+  if (id_x)
+    for (int j = 0; j < k; ++j)
+      if (ids[t * k + j] >= E) idw += wts[t * k + j];
   for (int c = threadIdx.x; c < H; c += blockDim.x) {
     float a = add ? ldv(add + t * add_stride + c) : 0.f;
     for (int j = 0; j < k; ++j) {
       const int p = inv[t * k + j];
       if (p >= 0) a += ldv(y + (int64_t)p * H + c);
     }
+    if (idw != 0.f) a += idw * ldv(id_x + t * id_stride + c);
     stv(out + t * H + c, a);
   }
 }
@@ -558,6 +656,21 @@ void launch_moe_route_scores(const float* logits, int64_t ld, int T, int E, int 
   moe_route_scores_kernel<<<(T + 127) / 128, 128, 0, stream>>>(logits, ld, T, E, k, score, renorm ? 1 : 0, ids, w);
 }
 
+void launch_moe_route_grouped(const float* logits, int64_t ld, const float* correction, int T, int E, int k, int groups,
+                              int keep, float scale, int32_t* ids, float* w, hipStream_t stream) {
+  if (T == 0) return;
+  if (E > RG_MAX_E || groups > RG_MAX_GROUPS) abort();   // the binding checks both
+  const size_t smem = (size_t)2 * E * RG_THREADS * sizeof(float);
+  static bool attr_set = false;
+  if (smem > 65536 && !attr_set) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_route_grouped_kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    attr_set = true;
+  }
+  moe_route_grouped_kernel<<<(T + RG_THREADS - 1) / RG_THREADS, RG_THREADS, smem, stream>>>(logits, ld, correction, T, E, k,
+                                                                                           groups, keep, scale, ids, w);
+}
+
 void launch_moe_gemm_rows(const MoeRowsParams& p, int mode, bool f32, hipStream_t stream) {
   const int N = mode == 0 ? p.F : p.N;
   if (p.mt == 0 || N == 0) return;
@@ -572,21 +685,25 @@ void launch_moe_gemm_rows(const MoeRowsParams& p, int mode, bool f32, hipStream_
 }
 
 void launch_moe_combine_rows(const void* y, const int32_t* inv, int T, int k, int H, const void* add,
-                             int64_t add_stride, void* out, bool f32, hipStream_t stream) {
+                             int64_t add_stride, void* out, const void* id_x, int64_t id_stride, const int32_t* ids,
+                             const float* wts, int E, bool f32, hipStream_t stream) {
   if (T == 0) return;
-  if (!f32 && H % 8 == 0 && (add == nullptr || (add_stride % 8 == 0 && ((uintptr_t)add % 16) == 0))) {
+  if (!f32 && H % 8 == 0 && (add == nullptr || (add_stride % 8 == 0 && ((uintptr_t)add % 16) == 0)) &&
+      (id_x == nullptr || (id_stride % 8 == 0 && ((uintptr_t)id_x % 16) == 0))) {
     int64_t g = ((int64_t)T * H / 8 + 255) / 256;
     if (g > 4096) g = 4096;
     moe_combine_kernel<<<(unsigned)g, 256, 0, stream>>>((const uint16_t*)y, inv, T, k, H, (uint16_t*)out,
-                                                        (const uint16_t*)add, add_stride);
+                                                        (const uint16_t*)add, add_stride, (const uint16_t*)id_x,
+                                                        id_stride, ids, wts, E);
     return;
   }
   if (f32)
     moe_combine_rows_kernel<float><<<T, 256, 0, stream>>>((const float*)y, inv, k, H, (const float*)add, add_stride,
-                                                         (float*)out);
+                                                         (float*)out, (const float*)id_x, id_stride, ids, wts, E);
   else
     moe_combine_rows_kernel<uint16_t><<<T, 256, 0, stream>>>((const uint16_t*)y, inv, k, H, (const uint16_t*)add,
-                                                            add_stride, (uint16_t*)out);
+                                                            add_stride, (uint16_t*)out, (const uint16_t*)id_x, id_stride,
+                                                            ids, wts, E);
 }
 
 void launch_moe_combine(const uint16_t* y, const int32_t* inv, int T, int k, int H, uint16_t* out,

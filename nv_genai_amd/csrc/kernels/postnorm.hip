@@ -14,9 +14,15 @@
 //   softcap           z = cap * tanh(z * scale / cap) on fp32 logits
 //   residual_add_rmsnorm   x[t] += y[t], out[t] = rmsnorm(x[t]) * w: the residual sum of one
 //                     pre-norm sub-layer and the norm in front of the next in one pass
-//   clamped_glu       [gate F | up F | ...] -> g sigmoid(alpha g) (u + 1), g = min(gate, limit),
+//   clamped_glu       [gate F | up F | ...] -> g sigmoid(alpha g) (u + shift), g = min(gate, limit),
 //                     u = clamp(up, +-limit), optionally times sigmoid of one gate column of the row
-//   group_rmsnorm     RMS norm of each of G equal column groups of fp32 rows (heads)
+//   group_rmsnorm     RMS norm of each of G equal column groups of fp32 rows (heads), weight per
+//                     group element or per column, optional sigmoid gate per column
+//   dyt_norm          tanh(alpha x) * w + b of fp32 rows (dynamic tanh in place of a norm)
+//   residual_dyt      x += (y1 + y2 + bias), or x = y1, and the dynamic tanh of the result:
+//                     the step between two parallel layers in one pass
+//   pack_pair         [a | b] rows of two fp32 streams in the activation type
+//   bias_gelu_tanh    gelu_tanh(x + bias) in place, fp32 bias, any width
 //
 // The residual, the norms and the shift interpolation are fp32 whatever the activation type T
 // (bf16 storage as uint16_t, or float). Memory-bound: one workgroup per row, columns strided
@@ -213,7 +219,7 @@ __global__ void __launch_bounds__(256) residual_add_rmsnorm_kernel(float* __rest
 template <typename T>
 __global__ void __launch_bounds__(256) clamped_glu_kernel(T* __restrict__ out, const T* __restrict__ in,
                                                           int64_t in_stride, int64_t T_rows, int F, float limit,
-                                                          float alpha, int gate_col) {
+                                                          float alpha, int gate_col, float shift) {
   const int64_t total = T_rows * F;
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t t = i / F;
@@ -221,7 +227,7 @@ __global__ void __launch_bounds__(256) clamped_glu_kernel(T* __restrict__ out, c
     const T* r = in + t * in_stride;
     const float g = fminf(ldf(r + c), limit);
     const float u = fminf(fmaxf(ldf(r + F + c), -limit), limit);
-    float v = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+    float v = g / (1.0f + expf(-alpha * g)) * (u + shift);
     if (gate_col >= 0) v *= 1.0f / (1.0f + expf(-ldf(r + gate_col)));
     stf(out + i, v);
   }
@@ -230,7 +236,7 @@ __global__ void __launch_bounds__(256) clamped_glu_kernel(T* __restrict__ out, c
 // bf16 rows with F % 8 == 0 and 16-byte aligned rows: 8 gates and 8 ups per thread
 __global__ void __launch_bounds__(256) clamped_glu_bf16x8_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ in,
                                                                  int64_t in_stride, int64_t T_rows, int F8, float limit,
-                                                                 float alpha, int gate_col) {
+                                                                 float alpha, int gate_col, float shift) {
   const int64_t total = T_rows * F8;
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t t = i / F8;
@@ -243,7 +249,7 @@ __global__ void __launch_bounds__(256) clamped_glu_bf16x8_kernel(uint16_t* __res
     for (int j = 0; j < 8; ++j) {
       const float g = fminf(bf2f(g8[j]), limit);
       const float u = fminf(fmaxf(bf2f(u8[j]), -limit), limit);
-      o[j] = f2bf(g / (1.0f + expf(-alpha * g)) * (u + 1.0f) * rg);
+      o[j] = f2bf(g / (1.0f + expf(-alpha * g)) * (u + shift) * rg);
     }
     store8(out + t * 8 * F8 + c, o);
   }
@@ -255,19 +261,101 @@ __global__ void __launch_bounds__(256) softcap_kernel(float* __restrict__ z, int
 }
 
 // one wave per (row, group)
+// w_groups: groups per row when every column has its own weight (else 0: gs weights shared by
+// the groups); gate: rows [groups * gs] of the output type with stride g_stride, sigmoid applied
 template <typename T>
 __global__ void __launch_bounds__(256) group_rmsnorm_kernel(T* __restrict__ out, const float* __restrict__ x,
                                                             const float* __restrict__ w, int64_t n_groups, int gs,
-                                                            float eps) {
+                                                            float eps, int groups, int w_full,
+                                                            const T* __restrict__ gate, int64_t g_stride) {
   const int64_t g = blockIdx.x * (int64_t)(blockDim.x >> 6) + (threadIdx.x >> 6);
   if (g >= n_groups) return;
   const int lane = threadIdx.x & 63;
   const float* xr = x + g * gs;
+  const int64_t row = g / groups;
+  const int hg = (int)(g - row * groups);
+  const float* wr = w_full ? w + (int64_t)hg * gs : w;
+  const T* gr = gate ? gate + row * g_stride + (int64_t)hg * gs : nullptr;
   float ss = 0.f;
   for (int c = lane; c < gs; c += 64) ss += xr[c] * xr[c];
   ss = wave_sum(ss);
   const float r = 1.0f / sqrtf(ss / (float)gs + eps);
-  for (int c = lane; c < gs; c += 64) stf(out + g * gs + c, xr[c] * r * w[c]);
+  for (int c = lane; c < gs; c += 64) {
+    float v = xr[c] * r * wr[c];
+    if (gr) v *= 1.0f / (1.0f + expf(-ldf(gr + c)));
+    stf(out + g * gs + c, v);
+  }
+}
+
+// ---- dynamic tanh in place of a norm: tanh(alpha x) * w + b, no statistics
+// rows: gather (nullptr: all rows)
+template <typename T>
+__global__ void __launch_bounds__(256) dyt_norm_kernel(T* __restrict__ out, const float* __restrict__ x, float alpha,
+                                                       const float* __restrict__ w, const float* __restrict__ b,
+                                                       const int64_t* __restrict__ rows, int H) {
+  const int64_t r = blockIdx.x;
+  const float* xr = x + (rows ? rows[r] : r) * H;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) stf(out + r * H + c, tanhf(alpha * xr[c]) * w[c] + b[c]);
+}
+
+// x += (y1 + y2 + bias) (fp32 sums), or x = y1 (assign); out = tanh(alpha x) * w + b
+template <typename T>
+__global__ void __launch_bounds__(256) residual_dyt_kernel(float* __restrict__ x, const T* __restrict__ y1, int64_t s1,
+                                                           const T* __restrict__ y2, int64_t s2,
+                                                           const float* __restrict__ bias, float alpha,
+                                                           const float* __restrict__ w, const float* __restrict__ b,
+                                                           T* __restrict__ out, int H, int assign) {
+  const int64_t r = blockIdx.x;
+  float* xr = x + r * H;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    float y = ldf(y1 + r * s1 + c);
+    if (y2) y += ldf(y2 + r * s2 + c);
+    if (bias) y += bias[c];
+    const float v = assign ? y : xr[c] + y;
+    xr[c] = v;
+    if (out) stf(out + r * H + c, tanhf(alpha * v) * w[c] + b[c]);
+  }
+}
+
+// out row = [a row | b row] in the activation type
+template <typename T>
+__global__ void __launch_bounds__(256) pack_pair_kernel(T* __restrict__ out, const float* __restrict__ a,
+                                                        const float* __restrict__ b, int Ha, int Hb) {
+  const int64_t r = blockIdx.x;
+  T* o = out + r * (Ha + Hb);
+  for (int c = threadIdx.x; c < Ha; c += blockDim.x) stf(o + c, a[r * Ha + c]);
+  for (int c = threadIdx.x; c < Hb; c += blockDim.x) stf(o + Ha + c, b[r * Hb + c]);
+}
+
+// x = gelu_tanh(x + bias) in place, any width
+template <typename T>
+__global__ void __launch_bounds__(256) bias_gelu_tanh_kernel(T* __restrict__ x, const float* __restrict__ bias,
+                                                             int64_t T_rows, int F) {
+  const int64_t total = T_rows * F;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int c = (int)(i % F);
+    const float z = ldf(x + i) + (bias ? bias[c] : 0.f);
+    stf(x + i, 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))));
+  }
+}
+
+// bf16 rows with F % 8 == 0: 8 elements per thread
+__global__ void __launch_bounds__(256) bias_gelu_tanh_bf16x8_kernel(uint16_t* __restrict__ x, const float* __restrict__ bias,
+                                                                    int64_t T_rows, int F8) {
+  const int64_t total = T_rows * F8;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int c = (int)(i % F8) * 8;
+    const u16x8 v = load8(x + i * 8);
+    u16x8 o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float z = bf2f(v[j]) + (bias ? bias[c + j] : 0.f);
+      const float u = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+      // 0.5 z (1 + tanh u) = z - z / (1 + e^(2u))
+      o[j] = f2bf(z - z * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(2.8853900817779268f * u)));
+    }
+    store8(x + i * 8, o);
+  }
 }
 
 }  // namespace
@@ -384,34 +472,82 @@ void launch_residual_add_rmsnorm(float* x, const void* y, int64_t y_stride, cons
 }
 
 void launch_clamped_glu(void* out, const void* in, int64_t in_stride, int64_t T, int F, float limit, float alpha,
-                        int gate_col, bool f32, hipStream_t stream) {
+                        int gate_col, float shift, bool f32, hipStream_t stream) {
   if (T == 0 || F == 0) return;
   if (!f32 && F % 8 == 0 && in_stride % 8 == 0 && ((uintptr_t)in % 16) == 0 && ((uintptr_t)out % 16) == 0) {
     int64_t g8 = (T * (F / 8) + 255) / 256;
     if (g8 > 16384) g8 = 16384;
     clamped_glu_bf16x8_kernel<<<dim3((unsigned)g8), 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)in, in_stride, T,
-                                                                      F / 8, limit, alpha, gate_col);
+                                                                      F / 8, limit, alpha, gate_col, shift);
     return;
   }
   int64_t g = (T * F + 255) / 256;
   if (g > 8192) g = 8192;
   if (f32)
     clamped_glu_kernel<float><<<dim3((unsigned)g), 256, 0, stream>>>((float*)out, (const float*)in, in_stride, T, F,
-                                                                    limit, alpha, gate_col);
+                                                                    limit, alpha, gate_col, shift);
   else
     clamped_glu_kernel<uint16_t><<<dim3((unsigned)g), 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)in, in_stride,
-                                                                       T, F, limit, alpha, gate_col);
+                                                                       T, F, limit, alpha, gate_col, shift);
 }
 
-void launch_group_rmsnorm(void* out, const float* x, const float* w, int64_t T, int groups, int gs, float eps, bool f32,
-                          hipStream_t stream) {
+void launch_group_rmsnorm(void* out, const float* x, const float* w, bool w_full, const void* gate, int64_t g_stride,
+                          int64_t T, int groups, int gs, float eps, bool f32, hipStream_t stream) {
   const int64_t ng = T * groups;
   if (ng == 0) return;
   const unsigned g = (unsigned)((ng + 3) / 4);
   if (f32)
-    group_rmsnorm_kernel<float><<<dim3(g), 256, 0, stream>>>((float*)out, x, w, ng, gs, eps);
+    group_rmsnorm_kernel<float><<<dim3(g), 256, 0, stream>>>((float*)out, x, w, ng, gs, eps, groups, w_full ? 1 : 0,
+                                                             (const float*)gate, g_stride);
   else
-    group_rmsnorm_kernel<uint16_t><<<dim3(g), 256, 0, stream>>>((uint16_t*)out, x, w, ng, gs, eps);
+    group_rmsnorm_kernel<uint16_t><<<dim3(g), 256, 0, stream>>>((uint16_t*)out, x, w, ng, gs, eps, groups, w_full ? 1 : 0,
+                                                                (const uint16_t*)gate, g_stride);
+}
+
+void launch_dyt_norm(void* out, const float* x, float alpha, const float* w, const float* b, const int64_t* rows,
+                     int64_t n_out, int H, bool f32, hipStream_t stream) {
+  if (n_out == 0) return;
+  if (f32)
+    dyt_norm_kernel<float><<<dim3((unsigned)n_out), 256, 0, stream>>>((float*)out, x, alpha, w, b, rows, H);
+  else
+    dyt_norm_kernel<uint16_t><<<dim3((unsigned)n_out), 256, 0, stream>>>((uint16_t*)out, x, alpha, w, b, rows, H);
+}
+
+void launch_residual_dyt(float* x, const void* y1, int64_t s1, const void* y2, int64_t s2, const float* bias, float alpha,
+                         const float* w, const float* b, void* out, int64_t T, int H, bool assign, bool f32,
+                         hipStream_t stream) {
+  if (T == 0) return;
+  if (f32)
+    residual_dyt_kernel<float><<<dim3((unsigned)T), 256, 0, stream>>>(x, (const float*)y1, s1, (const float*)y2, s2, bias,
+                                                                     alpha, w, b, (float*)out, H, assign ? 1 : 0);
+  else
+    residual_dyt_kernel<uint16_t><<<dim3((unsigned)T), 256, 0, stream>>>(x, (const uint16_t*)y1, s1, (const uint16_t*)y2,
+                                                                        s2, bias, alpha, w, b, (uint16_t*)out, H,
+                                                                        assign ? 1 : 0);
+}
+
+void launch_pack_pair(void* out, const float* a, const float* b, int64_t T, int Ha, int Hb, bool f32, hipStream_t stream) {
+  if (T == 0) return;
+  if (f32)
+    pack_pair_kernel<float><<<dim3((unsigned)T), 256, 0, stream>>>((float*)out, a, b, Ha, Hb);
+  else
+    pack_pair_kernel<uint16_t><<<dim3((unsigned)T), 256, 0, stream>>>((uint16_t*)out, a, b, Ha, Hb);
+}
+
+void launch_bias_gelu_tanh(void* x, const float* bias, int64_t T, int F, bool f32, hipStream_t stream) {
+  if (T == 0 || F == 0) return;
+  if (!f32 && F % 8 == 0 && ((uintptr_t)x % 16) == 0) {
+    int64_t g8 = (T * (F / 8) + 255) / 256;
+    if (g8 > 16384) g8 = 16384;
+    bias_gelu_tanh_bf16x8_kernel<<<dim3((unsigned)g8), 256, 0, stream>>>((uint16_t*)x, bias, T, F / 8);
+    return;
+  }
+  int64_t g = (T * F + 255) / 256;
+  if (g > 8192) g = 8192;
+  if (f32)
+    bias_gelu_tanh_kernel<float><<<dim3((unsigned)g), 256, 0, stream>>>((float*)x, bias, T, F);
+  else
+    bias_gelu_tanh_kernel<uint16_t><<<dim3((unsigned)g), 256, 0, stream>>>((uint16_t*)x, bias, T, F);
 }
 
 }  // namespace nga

@@ -4,6 +4,14 @@
 //                (a prompt portion, or a single decode row), with q = silu(q_pre) and
 //                f = lower + (1 - lower) * sigmoid(f_pre + f_bias) formed in fp32 in the kernel.
 //
+//   mlstm_scan   per head a matrix memory with exponential gates kept stable by a running maximum m:
+//                m' = max(f + m, i), S <- e^(f + m - m') S + e^(i - m') k v^T, n likewise with k,
+//                o = S^T q / (max(|n . q|, e^(-m')) + 1e-6), with the log gates
+//                i = cap tanh((i_pre + b) / cap), f = logsigmoid(cap tanh((f_pre + b) / cap)) and
+//                q scaled by d^(-1/2), all formed in fp32 in the kernel. Same tiling as hgrn2_scan;
+//                the gate chain of a pass (m, both decays, e^(-m)) is run once per pass by one
+//                lane and shared through LDS, the normaliser n is kept beside S in registers.
+//
 // A workgroup owns (segment, head, tile of VT value columns): thread (rg, j) keeps the state
 // elements S[rg * NR + k][j] in registers for the whole segment, so the state is read from its
 // slot once and written back once. Rows are staged through LDS TC at a time: the raw values of the
@@ -192,7 +200,223 @@ bool launch_hgrn2_t(float* out, const T* proj, int64_t stride, const float* f_bi
 #undef NGA_HGRN2_ARGS
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// mLSTM. proj row: q [H*d] at q_off, k [H*d] at k_off, v [H*dv] at v_off, gate pre-activations
+// [i (H) | f (H)] at g_off. State slot of a head: S [d][dv], n [d], m (d * dv + d + 1 floats).
+// cu == nullptr: segment b is row b. Padded state rows (i >= d) see k = q = 0 and stay 0.
+__device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+template <typename T, int NR, int VT>
+__global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out, const T* __restrict__ proj,
+                                                         int64_t stride, const float* __restrict__ gate_bias,
+                                                         float* __restrict__ state, int H, int d, int dv, float cap,
+                                                         const int32_t* __restrict__ cu,
+                                                         const int32_t* __restrict__ slots,
+                                                         const int32_t* __restrict__ pos, int q_off, int k_off,
+                                                         int v_off, int g_off) {
+  constexpr int RG = 256 / VT;
+  constexpr int DP = RG * NR;              // padded rows of a head
+  constexpr int NQ = TC * DP / 256;        // q (and k) elements a thread stages per pass
+  constexpr int NV = (TC * VT + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float qs[TC * DP];
+  __shared__ __attribute__((aligned(16))) float ks[TC * DP];
+  __shared__ float vs[TC * VT];
+  __shared__ float part[TC * 256];
+  __shared__ float partn[TC * RG];
+  __shared__ float gi[TC], gf[TC];         // log gates of the pass
+  __shared__ float ga[TC], gb[TC], gem[TC];   // decay of the old state, weight of the new row, e^(-m)
+  __shared__ float m_carry;
+  const int vt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int t0 = cu ? cu[b] : b, t1 = cu ? cu[b + 1] : b + 1;
+  if (t1 <= t0) return;
+  const int slot = slots[b];
+  const bool fresh = slot < 0 || pos[t0] == 0;
+  const int tid = threadIdx.x;
+  const int j = tid % VT, rg = tid / VT;
+  const int col = vt * VT + j;
+  const bool colok = col < dv;
+  const int64_t ssz = (int64_t)d * dv + d + 1;
+  float* sp = slot >= 0 ? state + ((int64_t)slot * H + h) * ssz : nullptr;
+  float S[NR], n[NR];
+#pragma unroll
+  for (int k = 0; k < NR; ++k) {
+    const int i = rg * NR + k;
+    const bool ld = !fresh && i < d;
+    S[k] = (ld && colok) ? sp[(int64_t)i * dv + col] : 0.f;
+    n[k] = ld ? sp[(int64_t)d * dv + i] : 0.f;
+  }
+  if (tid == 0) m_carry = fresh ? 0.f : sp[(int64_t)d * dv + d];
+  const float qscale = 1.0f / sqrtf((float)d);
+  const float inv_cap = 1.0f / cap;
+  const int qo = q_off + h * d, ko = k_off + h * d, vo = v_off + h * dv + vt * VT;
+  float rq[NQ], rk[NQ], rv[NV], ri = 0.f, rf = 0.f;
+  // raw values of rows [tc, tc + TC) into registers (rows past t1 and padded columns: zeros)
+  auto fetch = [&](int tc) {
+#pragma unroll
+    for (int x = 0; x < NQ; ++x) {
+      const int e = tid + 256 * x, tt = e / DP, i = e % DP;
+      const bool ok = tc + tt < t1 && i < d;
+      const T* pr = proj + (int64_t)(tc + tt) * stride;
+      rq[x] = ok ? ldf(pr + qo + i) : 0.f;
+      rk[x] = ok ? ldf(pr + ko + i) : 0.f;
+    }
+#pragma unroll
+    for (int x = 0; x < NV; ++x) {
+      const int e = tid + 256 * x, tt = e / VT, jj = e % VT;
+      rv[x] = (e < TC * VT && tc + tt < t1 && vt * VT + jj < dv) ? ldf(proj + (int64_t)(tc + tt) * stride + vo + jj) : 0.f;
+    }
+    if (tid < TC && tc + tid < t1) {
+      const T* pr = proj + (int64_t)(tc + tid) * stride + g_off;
+      ri = ldf(pr + h);
+      rf = ldf(pr + H + h);
+    }
+  };
+  fetch(t0);
+  for (int tc = t0; tc < t1; tc += TC) {
+    const int nt = t1 - tc < TC ? t1 - tc : TC;
+    __syncthreads();   // the previous pass is done with the staged rows, part / partn and the gate chain
+#pragma unroll
+    for (int x = 0; x < NQ; ++x) {
+      const int e = tid + 256 * x;
+      qs[e] = rq[x] * qscale;
+      ks[e] = rk[x];
+    }
+#pragma unroll
+    for (int x = 0; x < NV; ++x) {
+      const int e = tid + 256 * x;
+      if (e < TC * VT) vs[e] = rv[x];
+    }
+    if (tid < TC) {
+      gi[tid] = cap * tanhf((ri + gate_bias[h]) * inv_cap);
+      gf[tid] = log_sigmoid(cap * tanhf((rf + gate_bias[H + h]) * inv_cap));
+    }
+    __syncthreads();
+    if (tid == 0) {   // the gate chain of the pass: sequential, a few exponentials per row
+      float m = m_carry;
+      for (int tt = 0; tt < nt; ++tt) {
+        const float fm = gf[tt] + m;
+        const float mn = fmaxf(fm, gi[tt]);
+        ga[tt] = expf(fm - mn);
+        gb[tt] = expf(gi[tt] - mn);
+        gem[tt] = expf(-mn);
+        m = mn;
+      }
+      m_carry = m;
+    }
+    __syncthreads();
+    if (tc + TC < t1) fetch(tc + TC);   // lands while this pass computes
+    auto row = [&](int tt) {
+      const float a = ga[tt];
+      const float bv = gb[tt] * vs[tt * VT + j], bb = gb[tt];
+      const float4* kr = reinterpret_cast<const float4*>(ks + tt * DP + rg * NR);
+      const float4* qr = reinterpret_cast<const float4*>(qs + tt * DP + rg * NR);
+      float p = 0.f, pn = 0.f;
+#pragma unroll
+      for (int k4 = 0; k4 < NR / 4; ++k4) {
+        const float4 k4v = kr[k4], q4 = qr[k4];
+        const float ka[4] = {k4v.x, k4v.y, k4v.z, k4v.w}, qa[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int k = 4 * k4 + u;
+          S[k] = a * S[k] + ka[u] * bv;
+          n[k] = a * n[k] + ka[u] * bb;
+          p += S[k] * qa[u];
+          pn += n[k] * qa[u];
+        }
+      }
+      part[tt * 256 + tid] = p;
+      if (j == 0) partn[tt * RG + rg] = pn;
+    };
+    if (nt == TC) {   // full pass: unrolled, so the LDS reads of later rows run ahead of the recurrence
+#pragma unroll
+      for (int tt = 0; tt < TC; ++tt) row(tt);
+    } else {
+      for (int tt = 0; tt < nt; ++tt) row(tt);
+    }
+    __syncthreads();
+    for (int e = tid; e < nt * VT; e += 256) {
+      const int tt = e / VT, jj = e % VT;
+      if (vt * VT + jj < dv) {
+        float s2 = 0.f, nq = 0.f;
+#pragma unroll
+        for (int r = 0; r < RG; ++r) {
+          s2 += part[tt * 256 + r * VT + jj];
+          nq += partn[tt * RG + r];
+        }
+        out[(int64_t)(tc + tt) * H * dv + h * dv + vt * VT + jj] = s2 / (fmaxf(fabsf(nq), gem[tt]) + 1e-6f);
+      }
+    }
+  }
+  if (sp) {
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
+      const int i = rg * NR + k;
+      if (i < d) {
+        if (colok) sp[(int64_t)i * dv + col] = S[k];
+        if (vt == 0 && j == 0) sp[(int64_t)d * dv + i] = n[k];
+      }
+    }
+    __syncthreads();   // m_carry of the last pass
+    if (vt == 0 && tid == 0) sp[(int64_t)d * dv + d] = m_carry;
+  }
+}
+
+template <typename T, int VT>
+bool launch_mlstm_vt(float* out, const T* proj, int64_t stride, const float* gate_bias, float* state, int H, int d,
+                     int dv, float cap, const int32_t* cu, const int32_t* slots, const int32_t* pos, int n_seg, int q_off,
+                     int k_off, int v_off, int g_off, hipStream_t stream) {
+  constexpr int RG = 256 / VT;
+  const int nr = (d + RG - 1) / RG;
+  const dim3 grid((unsigned)((dv + VT - 1) / VT), (unsigned)H, (unsigned)n_seg);
+#define NGA_MLSTM_CASE(N)                                                                                            \
+  if (nr <= N) {                                                                                                     \
+    mlstm_scan_kernel<T, N, VT><<<grid, 256, 0, stream>>>(out, proj, stride, gate_bias, state, H, d, dv, cap, cu, slots, \
+                                                          pos, q_off, k_off, v_off, g_off);                          \
+    return true;                                                                                                     \
+  }
+  // at most 256 padded rows per head in LDS: NR <= 64 / 32 / 16 for tiles of 64 / 32 / 16 columns
+  NGA_MLSTM_CASE(4)
+  NGA_MLSTM_CASE(8)
+  NGA_MLSTM_CASE(16)
+  if constexpr (VT >= 32) {
+    NGA_MLSTM_CASE(32)
+  }
+  if constexpr (VT >= 64) {
+    NGA_MLSTM_CASE(64)
+  }
+#undef NGA_MLSTM_CASE
+  return false;
+}
+
+template <typename T>
+bool launch_mlstm_t(float* out, const T* proj, int64_t stride, const float* gate_bias, float* state, int H, int d, int dv,
+                    float cap, const int32_t* cu, const int32_t* slots, const int32_t* pos, int n_seg, int q_off,
+                    int k_off, int v_off, int g_off, hipStream_t stream) {
+  const int64_t base = (int64_t)n_seg * H;
+  int vt = dv <= 16 ? 16 : (dv <= 32 ? 32 : 64);
+  while (vt > 16 && base * ((dv + vt - 1) / vt) < 1024) vt /= 2;
+#define NGA_MLSTM_ARGS out, proj, stride, gate_bias, state, H, d, dv, cap, cu, slots, pos, n_seg, q_off, k_off, v_off, g_off, stream
+  if (vt == 64 && launch_mlstm_vt<T, 64>(NGA_MLSTM_ARGS)) return true;
+  if (vt >= 32 && launch_mlstm_vt<T, 32>(NGA_MLSTM_ARGS)) return true;
+  return launch_mlstm_vt<T, 16>(NGA_MLSTM_ARGS);
+#undef NGA_MLSTM_ARGS
+}
+
 }  // namespace
+
+int mlstm_max_dim() { return 256; }   // padded rows of a head that fit the LDS staging
+
+bool launch_mlstm_scan(float* out, const void* proj, int64_t stride, const float* gate_bias, float* state, int H, int d,
+                       int dv, float cap, const int32_t* cu, const int32_t* slots, const int32_t* pos, int n_seg,
+                       int q_off, int k_off, int v_off, int g_off, bool f32, hipStream_t stream) {
+  if (n_seg == 0) return true;
+  if (f32)
+    return launch_mlstm_t<float>(out, (const float*)proj, stride, gate_bias, state, H, d, dv, cap, cu, slots, pos, n_seg,
+                                 q_off, k_off, v_off, g_off, stream);
+  return launch_mlstm_t<uint16_t>(out, (const uint16_t*)proj, stride, gate_bias, state, H, d, dv, cap, cu, slots, pos,
+                                  n_seg, q_off, k_off, v_off, g_off, stream);
+}
 
 int hgrn2_max_dim(int dv) { return 256; }   // padded rows of a head that fit the LDS staging
 

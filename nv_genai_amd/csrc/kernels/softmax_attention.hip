@@ -126,7 +126,7 @@ __global__ void __launch_bounds__(64) softmax_attention_kernel(
     T* __restrict__ out, const T* __restrict__ q, int64_t q_stride, const T* __restrict__ gate, int64_t g_stride,
     const T* __restrict__ kc, const T* __restrict__ vc, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int H, int G, int dk, int dv, float scale,
-    int window, int maps, float lam, float unit_eps, float out_scale, int v_row) {
+    int window, int maps, float lam, float unit_eps, float out_scale, int v_row, float softcap) {
   extern __shared__ float smem[];
   float* qs = smem;                 // [maps * dk]
   float* ws = smem + maps * dk;     // [64]
@@ -161,7 +161,10 @@ __global__ void __launch_bounds__(64) softmax_attention_kernel(
       const bool vis = j >= lo && j <= i;
       const int64_t page = bt[p];
       float s = -INFINITY;
-      if (vis) s = dot_row(qs + m * dk, kc + ((page * G * maps + kh) * BS + lane) * (int64_t)dk, dk, vec) * scale;
+      if (vis) {
+        s = dot_row(qs + m * dk, kc + ((page * G * maps + kh) * BS + lane) * (int64_t)dk, dk, vec) * scale;
+        if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+      }
       const float nmx = fmaxf(mx, wave_max(s));   // every visited page holds a visible key
       const float corr = expf(mx - nmx);          // 0 on the first page (mx = -inf)
       const float w = vis ? expf(s - nmx) : 0.f;
@@ -216,6 +219,11 @@ __global__ void __launch_bounds__(64) softmax_attention_kernel(
 // lanes. The softmax runs per query column in the exp2 domain: the running maximum and sum are
 // reduced over the lane's 16 scores and the 4 lanes of its column; accumulators are rescaled
 // when the maximum moves. Pages visited: those the block's windows cover.
+// tanh on the hardware exp2 and reciprocal (soft cap of the scores in the MFMA kernels)
+__device__ __forceinline__ float tanh_fast(float x) {
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(2.8853900817779268f * x));
+}
+
 __device__ __forceinline__ int sm_row_swz(int row) { return (row & 3) | (((row >> 3) & 3) << 2); }
 
 struct SmMfmaParams {
@@ -230,6 +238,7 @@ struct SmMfmaParams {
   int64_t q_stride, g_stride;
   int max_blocks, H, G, window;
   float scale_log2, lam, unit_eps, out_scale;
+  float cap_log2;            // soft cap of the scores times log2 e (0: none)
   int v_row;                 // elements between value rows of a page (DV, or DK when the values lie in the key rows)
 };
 
@@ -366,6 +375,8 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
     const int kbase = t * KT;
     const float fd = (float)(qpos - kbase - 8 * h);
     const bool need_mask = kbase + KT - 1 > wq_lo || (W > 0 && wq_hi - kbase >= W);
+    const bool capped = P.cap_log2 > 0.f;
+    const float inv_cap = capped ? 1.0f / P.cap_log2 : 0.f;
     bf16x8 pf[MAPS][2];
     f32x4 sboth[SHARE ? MAPS : 1][4];
     if constexpr (SHARE) {   // both heads' scores from one read of every K fragment
@@ -409,6 +420,7 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
           float sv = sacc[tau][rr] * P.scale_log2;
+          if (capped) sv = P.cap_log2 * tanh_fast(sv * inv_cap);
           if (need_mask) {
             const float d = fd - (float)(32 * (tau >> 1) + 4 * (tau & 1) + rr);
             sv = (d >= 0.f && d < fW) ? sv : -INFINITY;
@@ -607,7 +619,7 @@ template <int DK, int DV, int MAPS>
 __device__ __forceinline__ void softmax_decode_mfma_body(
     float* __restrict__ ws, const uint16_t* __restrict__ q, int64_t q_stride, const uint16_t* __restrict__ kc,
     const uint16_t* __restrict__ vc, const int32_t* __restrict__ block_tables, int max_blocks,
-    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int H, int G, float scale_log2, int window,
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int H, int G, float scale_log2, float cap_log2, int window,
     int v_row) {
   constexpr int KT = 64;
   constexpr int DS = DK / 32;
@@ -685,6 +697,8 @@ __device__ __forceinline__ void softmax_decode_mfma_body(
     if (!have) continue;
     const int kbase = pg * KT;
     const bool need_mask = kbase < lo || kbase + KT - 1 > i;
+    const bool capped = cap_log2 > 0.f;
+    const float inv_cap = capped ? 1.0f / cap_log2 : 0.f;
     bf16x8 pf[MAPS][2];
 #pragma unroll
     for (int m = 0; m < MAPS; ++m) {
@@ -709,6 +723,7 @@ __device__ __forceinline__ void softmax_decode_mfma_body(
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
           float sv = sacc[tau][rr] * scale_log2;
+          if (capped) sv = cap_log2 * tanh_fast(sv * inv_cap);
           if (need_mask) {
             const int j = kbase + 32 * (tau >> 1) + 8 * h + 4 * (tau & 1) + rr;
             sv = (j >= lo && j <= i) ? sv : -INFINITY;
@@ -819,9 +834,9 @@ template <int DK, int DV, int MAPS>
 __global__ void __launch_bounds__(256) softmax_decode_mfma_kernel(
     float* __restrict__ ws, const uint16_t* __restrict__ q, int64_t q_stride, const uint16_t* __restrict__ kc,
     const uint16_t* __restrict__ vc, const int32_t* __restrict__ block_tables, int max_blocks,
-    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int H, int G, float scale_log2, int window,
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int H, int G, float scale_log2, float cap_log2, int window,
     int v_row) {
-  softmax_decode_mfma_body<DK, DV, MAPS>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2,
+  softmax_decode_mfma_body<DK, DV, MAPS>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, cap_log2,
                                          window, v_row);
 }
 
@@ -829,9 +844,9 @@ template <int DK, int DV, int MAPS>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) softmax_decode_mfma_kernel_w2(
     float* __restrict__ ws, const uint16_t* __restrict__ q, int64_t q_stride, const uint16_t* __restrict__ kc,
     const uint16_t* __restrict__ vc, const int32_t* __restrict__ block_tables, int max_blocks,
-    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int H, int G, float scale_log2, int window,
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int H, int G, float scale_log2, float cap_log2, int window,
     int v_row) {
-  softmax_decode_mfma_body<DK, DV, MAPS>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2,
+  softmax_decode_mfma_body<DK, DV, MAPS>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, cap_log2,
                                          window, v_row);
 }
 
@@ -882,7 +897,7 @@ __global__ void __launch_bounds__(64) softmax_decode_reduce_kernel(
 template <int DK, int DV, int MAPS>
 void launch_sm_decode_one(float* ws, const uint16_t* q, int64_t q_stride, const uint16_t* kc, const uint16_t* vc,
                           const int32_t* block_tables, int max_blocks, const int32_t* tok_seq, const int32_t* pos,
-                          int H, int G, float scale_log2, int window, int v_row, dim3 grid, hipStream_t stream) {
+                          int H, int G, float scale_log2, float cap_log2, int window, int v_row, dim3 grid, hipStream_t stream) {
   constexpr size_t tiles = (size_t)4 * DV * 64 * sizeof(uint16_t);
   constexpr size_t merge = (size_t)(4 * MAPS * 2 * 16 + MAPS * 16 * DV) * sizeof(float);
   constexpr size_t smem = tiles > merge ? tiles : merge;
@@ -894,7 +909,7 @@ void launch_sm_decode_one(float* ws, const uint16_t* q, int64_t q_stride, const 
       attr_set = true;
     }
     softmax_decode_mfma_kernel_w2<DK, DV, MAPS><<<grid, 256, smem, stream>>>(ws, q, q_stride, kc, vc, block_tables,
-                                                                            max_blocks, tok_seq, pos, H, G, scale_log2,
+                                                                            max_blocks, tok_seq, pos, H, G, scale_log2, cap_log2,
                                                                             window, v_row);
   } else {
     if (smem > 65536 && !attr_set) {
@@ -903,16 +918,16 @@ void launch_sm_decode_one(float* ws, const uint16_t* q, int64_t q_stride, const 
       attr_set = true;
     }
     softmax_decode_mfma_kernel<DK, DV, MAPS><<<grid, 256, smem, stream>>>(ws, q, q_stride, kc, vc, block_tables,
-                                                                         max_blocks, tok_seq, pos, H, G, scale_log2,
+                                                                         max_blocks, tok_seq, pos, H, G, scale_log2, cap_log2,
                                                                          window, v_row);
   }
 }
 
-#define NGA_SM_DEC_ARGS ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, window, v_row, grid, stream
+#define NGA_SM_DEC_ARGS ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, cap_log2, window, v_row, grid, stream
 template <int DK, int MAPS>
 bool launch_sm_decode_dv(float* ws, const uint16_t* q, int64_t q_stride, const uint16_t* kc, const uint16_t* vc,
                          const int32_t* block_tables, int max_blocks, const int32_t* tok_seq, const int32_t* pos, int H,
-                         int G, float scale_log2, int window, int v_row, int dv, dim3 grid, hipStream_t stream) {
+                         int G, float scale_log2, float cap_log2, int window, int v_row, int dv, dim3 grid, hipStream_t stream) {
   switch (dv) {
     case 32: launch_sm_decode_one<DK, 32, MAPS>(NGA_SM_DEC_ARGS); return true;
     case 64: launch_sm_decode_one<DK, 64, MAPS>(NGA_SM_DEC_ARGS); return true;
@@ -930,8 +945,8 @@ bool launch_sm_decode_dv(float* ws, const uint16_t* q, int64_t q_stride, const u
 template <int MAPS>
 bool launch_sm_decode_dk(float* ws, const uint16_t* q, int64_t q_stride, const uint16_t* kc, const uint16_t* vc,
                          const int32_t* block_tables, int max_blocks, const int32_t* tok_seq, const int32_t* pos, int H,
-                         int G, float scale_log2, int window, int v_row, int dk, int dv, dim3 grid, hipStream_t stream) {
-#define NGA_SM_DEC_DV(DKV) launch_sm_decode_dv<DKV, MAPS>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, window, v_row, dv, grid, stream)
+                         int G, float scale_log2, float cap_log2, int window, int v_row, int dk, int dv, dim3 grid, hipStream_t stream) {
+#define NGA_SM_DEC_DV(DKV) launch_sm_decode_dv<DKV, MAPS>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, cap_log2, window, v_row, dv, grid, stream)
   if (MAPS == 1) {   // key sizes of a latent plus a rotated part: one value size each
     if (dk == 96 && dv == 64) { launch_sm_decode_one<96, 64, 1>(NGA_SM_DEC_ARGS); return true; }
     if (dk == 192 && dv == 128) { launch_sm_decode_one<192, 128, 1>(NGA_SM_DEC_ARGS); return true; }
@@ -941,7 +956,7 @@ bool launch_sm_decode_dk(float* ws, const uint16_t* q, int64_t q_stride, const u
     case 32: return NGA_SM_DEC_DV(32);
     case 64: return NGA_SM_DEC_DV(64);
     case 128: return NGA_SM_DEC_DV(128);
-    case 256: return MAPS == 1 ? launch_sm_decode_dv<256, 1>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, window, v_row, dv, grid, stream) : false;
+    case 256: return MAPS == 1 ? launch_sm_decode_dv<256, 1>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, cap_log2, window, v_row, dv, grid, stream) : false;
     default: return false;
   }
 #undef NGA_SM_DEC_DV
@@ -968,16 +983,17 @@ void launch_softmax_decode_mfma(uint16_t* out, float* ws, int parts, const uint1
                                 const uint16_t* gate, int64_t g_stride, const uint16_t* kc, const uint16_t* vc,
                                 const int32_t* block_tables, int max_blocks, const int32_t* tok_seq,
                                 const int32_t* pos, int64_t T, int H, int G, int dk, int dv, float scale, int window,
-                                int maps, float lam, float unit_eps, float out_scale, bool v_in_k,
+                                int maps, float lam, float unit_eps, float out_scale, bool v_in_k, float softcap,
                                 hipStream_t stream) {
   if (T == 0) return;
   const dim3 grid((unsigned)parts, (unsigned)(G * ((H / G + 15) / 16)), (unsigned)T);
   const float scale_log2 = scale * 1.4426950408889634f;
+  const float cap_log2 = softcap > 0.f ? softcap * 1.4426950408889634f : 0.f;
   const int v_row = v_in_k ? dk : dv;
   const bool ok = maps == 2 ? launch_sm_decode_dk<2>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G,
-                                                     scale_log2, window, v_row, dk, dv, grid, stream)
+                                                     scale_log2, cap_log2, window, v_row, dk, dv, grid, stream)
                             : launch_sm_decode_dk<1>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G,
-                                                     scale_log2, window, v_row, dk, dv, grid, stream);
+                                                     scale_log2, cap_log2, window, v_row, dk, dv, grid, stream);
   if (!ok) abort();   // the caller checks softmax_attention_mfma_supported
   softmax_decode_reduce_kernel<<<dim3((unsigned)T, (unsigned)H), 64, 0, stream>>>(out, ws, parts, gate, g_stride, H,
                                                                                    dv, maps, lam, unit_eps, out_scale);
@@ -999,10 +1015,11 @@ void launch_softmax_attention_mfma(uint16_t* out, const uint16_t* q, int64_t q_s
                                    const int32_t* block_tables, int max_blocks, const int32_t* cu_q,
                                    const int32_t* ctx_lens, int B, int max_q_len, int H, int G, int dk, int dv,
                                    float scale, int window, int maps, float lam, float unit_eps, float out_scale,
-                                   bool v_in_k, hipStream_t stream) {
+                                   bool v_in_k, float softcap, hipStream_t stream) {
   if (B == 0 || max_q_len == 0) return;
   SmMfmaParams P{out, q, gate, kc, vc, block_tables, cu_q, ctx_lens, q_stride, g_stride, max_blocks, H, G, window,
-                 scale * 1.4426950408889634f, lam, unit_eps, out_scale, v_in_k ? dk : dv};
+                 scale * 1.4426950408889634f, lam, unit_eps, out_scale,
+                 softcap > 0.f ? softcap * 1.4426950408889634f : 0.f, v_in_k ? dk : dv};
   const dim3 grid((unsigned)H, (unsigned)B, (unsigned)((max_q_len + 63) / 64));   // (head, sequence, row block)
   const bool ok = maps == 2 ? launch_sm_mfma_dk<2>(P, dk, dv, grid, stream) : launch_sm_mfma_dk<1>(P, dk, dv, grid, stream);
   if (!ok) abort();   // the caller checks softmax_attention_mfma_supported
@@ -1026,7 +1043,7 @@ void launch_softmax_attention(void* out, const void* q, int64_t q_stride, const 
                               const void* kc, const void* vc, const int32_t* block_tables, int max_blocks,
                               const int32_t* tok_seq, const int32_t* pos, int64_t T, int H, int G, int dk, int dv,
                               float scale, int window, int maps, float lam, float unit_eps, float out_scale, bool v_in_k,
-                              bool f32, hipStream_t stream) {
+                              float softcap, bool f32, hipStream_t stream) {
   if (T == 0) return;
   const int v_row = v_in_k ? dk : dv;
   const dim3 grid((unsigned)T, (unsigned)H);
@@ -1034,12 +1051,13 @@ void launch_softmax_attention(void* out, const void* q, int64_t q_stride, const 
   if (f32)
     softmax_attention_kernel<float><<<grid, 64, smem, stream>>>(
         (float*)out, (const float*)q, q_stride, (const float*)gate, g_stride, (const float*)kc, (const float*)vc,
-        block_tables, max_blocks, tok_seq, pos, H, G, dk, dv, scale, window, maps, lam, unit_eps, out_scale, v_row);
+        block_tables, max_blocks, tok_seq, pos, H, G, dk, dv, scale, window, maps, lam, unit_eps, out_scale, v_row,
+        softcap);
   else
     softmax_attention_kernel<uint16_t><<<grid, 64, smem, stream>>>(
         (uint16_t*)out, (const uint16_t*)q, q_stride, (const uint16_t*)gate, g_stride, (const uint16_t*)kc,
         (const uint16_t*)vc, block_tables, max_blocks, tok_seq, pos, H, G, dk, dv, scale, window, maps, lam, unit_eps,
-        out_scale, v_row);
+        out_scale, v_row, softcap);
 }
 
 }  // namespace nga
