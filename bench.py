@@ -108,7 +108,7 @@ def parse(argv=None):
                     help="--workload designs: comma list of s, m, l (benchmarks/design_compare.py)")
     ap.add_argument("--design-models", default="bidasun",
                     help="--workload designs: comma list of the designs to run beside the closest Llama-layout model "
-                         "(bidasun, biruvik, lumepel)")
+                         "(bidasun, biruvik, lumepel, lizezen)")
     ap.add_argument("--workload", choices=("rag", "agent", "designs"), default="rag",
                     help="agent: query-decomposition agent, one TP=N replica + N-way sharded index")
     ap.add_argument("--kv-cache-fraction", type=float, default=None)

@@ -1,9 +1,10 @@
-"""The layer-list designs (Bidasun, Biruvik, Lumepel) beside the closest Llama-layout model at equal
-sizes (Mistral with a sliding window; Mixtral for Lumepel, whose feed-forwards are routed experts):
+"""The layer-list designs (Bidasun, Biruvik, Lumepel, Lizezen) beside the closest Llama-layout model at
+equal sizes (Mistral with a sliding window; Mixtral for Lumepel and Lizezen, whose feed-forwards are
+routed experts):
 prefill and decode throughput through the serving engine, and the design's kernels alone with
 their distance from the roofline. Random weights, synthetic token ids.
 
-    python bench.py --workload designs [--design-sizes s,m,l] [--design-models bidasun,biruvik,lumepel]
+    python bench.py --workload designs [--design-sizes s,m,l] [--design-models bidasun,biruvik,lumepel,lizezen]
 
 Prints one JSON line (``metric: design_compare``); bench.py's default workload is untouched.
 """
@@ -32,14 +33,26 @@ LUMEPEL = {"s": dict(rank=128, rot=64, q_rank=384, experts=8, top=2, eff=1024),
            "m": dict(rank=256, rot=64, q_rank=768, experts=16, top=2, eff=1408),
            "l": dict(rank=256, rot=64, q_rank=1536, experts=32, top=4, eff=2048)}
 LUMEPEL_PATTERN = ("latent_attention", "latent_attention_2")
-BASELINE_OF = {"bidasun": "mistral", "biruvik": "mistral", "lumepel": "mixtral"}
+# Lizezen: mLSTM heads of 64-wide keys and 128-wide values, rotary GQA attention with and without
+# head norms / score cap / head gate; every second feed-forward a mixture (expert sizes of LUMEPEL)
+# with two identity experts, four groups of which two are kept, and a shared expert
+LIZEZEN_PATTERN = ("mlstm", "attention", "mlstm", "attention_2")
+LIZEZEN_MLSTM = dict(dim=64, vdim=128)
+BASELINE_OF = {"bidasun": "mistral", "biruvik": "mistral", "lumepel": "mixtral", "lizezen": "mixtral"}
 
 
 def _engine(kind: str, z: dict, max_len: int, pages: int, seqs: int):
     from nv_genai_amd.engine.llm_engine import EngineConfig, LLMEngine
-    from nv_genai_amd.models.config import LlamaConfig, bidasun_uniform, biruvik_layers, lumepel_layers
+    from nv_genai_amd.models.config import LlamaConfig, bidasun_uniform, biruvik_layers, lizezen_layers, lumepel_layers
 
-    if kind == "lumepel":
+    if kind == "lizezen":
+        u = z["lumepel"]
+        pat = [LIZEZEN_PATTERN[i % len(LIZEZEN_PATTERN)] for i in range(z["layers"])]
+        mcfg = lizezen_layers(pat, z["hidden"], z["heads"], z["kv"], z["d"], z["d"], z["ffn"], mlstm_heads=z["heads"],
+                              mlstm_dim=LIZEZEN_MLSTM["dim"], mlstm_vdim=LIZEZEN_MLSTM["vdim"], experts=u["experts"] - 2,
+                              top=u["top"], expert_ff=u["eff"], shared_ff=u["eff"], identity=2, groups=4, keep=2,
+                              route_scale=2.5, softcap=30.0, rot_base=1e6, yarn=(8.0, 4096, 32.0, 1.0), vocab_size=VOCAB)
+    elif kind == "lumepel":
         u = z["lumepel"]
         pat = [LUMEPEL_PATTERN[i % len(LUMEPEL_PATTERN)] for i in range(z["layers"])]
         mcfg = lumepel_layers(pat, z["hidden"], z["heads"], z["d"], u["rot"], z["d"], u["rank"], u["q_rank"], 0,
@@ -359,6 +372,148 @@ def lumepel_kernel_times(z: dict, iters: int = 20) -> dict:
     return out
 
 
+def lizezen_kernel_times(z: dict, iters: int = 20) -> dict:
+    """The Lizezen kernels alone on one layer's shapes beside the like kernels of the other models:
+    the mLSTM scan against the HGRN2 scan (same state size), rotary GQA attention with head gate
+    and capped scores against causal softmax attention of the Llama layout, the group-routed SwiGLU
+    experts with identity experts against the Mixtral experts, and the row kernels (head norms +
+    rotation + page write against rotation + KV write; parallel residual step with the dynamic tanh
+    against residual sum + RMS norm; GELU with bias against the gated activation), priced by the
+    flops or bytes they must move."""
+    from nv_genai_amd import ops
+    from nv_genai_amd.ops import reference as ref
+
+    dev, bf = "cuda", torch.bfloat16
+    u = z["lumepel"]
+    H, G, D = z["heads"], z["kv"], z["d"]
+    d, dv = LIZEZEN_MLSTM["dim"], LIZEZEN_MLSTM["vdim"]
+    nb, L = z["pf"]
+    nd, ctx = z["dec"]
+    T = nb * L
+    out = {}
+    # ---- scans: prompts (nb segments of L rows) and single rows (nd segments)
+    nq, nv = H * d, H * dv
+    proj = torch.randn(T, 2 * nq + 2 * nv + 2 * H, device=dev).to(bf)
+    gb = torch.randn(2 * H, device=dev)
+    st = torch.zeros(max(nb, nd), H, ops.mlstm_state_size(d, dv), device=dev)
+    cu = torch.arange(0, T + 1, L, dtype=torch.int32, device=dev)
+    posr = torch.arange(L, dtype=torch.int32, device=dev).repeat(nb)
+    sl_p = torch.arange(nb, dtype=torch.int32, device=dev)
+    sl_d = torch.arange(nd, dtype=torch.int32, device=dev)
+    posd = torch.full((nd,), ctx - 1, dtype=torch.int32, device=dev)
+    offs = (0, nq, 2 * nq, 2 * nq + 2 * nv)
+    t_mp = _timed(lambda: ops.mlstm_scan(proj, gb, st, H, d, dv, 15.0, cu, sl_p, posr, offs), iters)
+    t_md = _timed(lambda: ops.mlstm_scan(proj[:nd], gb, st, H, d, dv, 15.0, None, sl_d, posd, offs), iters)
+    hp = torch.randn(T, 2 * nq + nv, device=dev).to(bf)
+    fb, lw = torch.randn(nq, device=dev), torch.rand(nq, device=dev) * 0.9
+    hs = torch.zeros(max(nb, nd), H, d, dv, device=dev)
+    t_hp = _timed(lambda: ops.hgrn2_scan(hp, fb, lw, hs, H, d, dv, cu, sl_p, posr), iters)
+    t_hd = _timed(lambda: ops.hgrn2_scan(hp[:nd], fb, lw, hs, H, d, dv, None, sl_d, posd), iters)
+    fl = 6.0 * T * H * d * dv                              # 3 FMAs per state element and row
+    by = nd * H * d * dv * 8.0                             # state read + written
+    out["scan"] = {"mlstm_prefill_ms": round(t_mp * 1e3, 3), "hgrn2_prefill_ms": round(t_hp * 1e3, 3),
+                   "mlstm_valu_frac": round(fl / t_mp / PEAK_VALU, 4), "hgrn2_valu_frac": round(fl / t_hp / PEAK_VALU, 4),
+                   "mlstm_decode_ms": round(t_md * 1e3, 4), "hgrn2_decode_ms": round(t_hd * 1e3, 4),
+                   "mlstm_state_hbm_frac": round(by / t_md / PEAK_HBM, 4), "hgrn2_state_hbm_frac": round(by / t_hd / PEAK_HBM, 4)}
+    del proj, hp
+    # ---- attention: capped scores and a head gate on row-major pages against the Llama-layout kernels
+    pages_seq = -(-max(L, ctx) // 64)
+    nseq = max(nb, nd)
+    npg = nseq * pages_seq
+    bt = torch.arange(npg, dtype=torch.int32, device=dev).view(nseq, pages_seq)
+    kr = (torch.randn(npg, G, 64, D, device=dev) * 0.5).to(bf)
+    vr = (torch.randn(npg, G, 64, D, device=dev) * 0.5).to(bf)
+    vt = (torch.randn(npg, G, D, 64, device=dev) * 0.5).to(bf)
+    cx = torch.full((nb,), L, dtype=torch.int32, device=dev)
+    q1 = torch.randn(T, H * D, device=dev).to(bf)
+    gate = torch.randn(T, H, device=dev).to(bf)
+    pairs = nb * (L * (L + 1) // 2) * H
+    sc = D ** -0.5
+    out["mfma_attention"] = bool(ops.softmax_attention_mfma_ok(q1, D, D, H // G, 1))
+    t_cap = _timed(lambda: ops.softmax_attention_prefill(q1, kr, vr, bt, cu, cx, L, H, G, D, D, sc, softcap=30.0, gate=gate),
+                   iters)
+    t_pl = _timed(lambda: ops.softmax_attention_prefill(q1, kr, vr, bt, cu, cx, L, H, G, D, D, sc), iters)
+    t_soft = _timed(lambda: ops.prefill_attention_paged(q1, kr, vt, bt, cu, cx, H, G, D, L, sc, window=0, impl=4), iters)
+    out["prefill"] = {"capped_gated_ms": round(t_cap * 1e3, 3), "plain_ms": round(t_pl * 1e3, 3),
+                      "llama_layout_ms": round(t_soft * 1e3, 3),
+                      "capped_gated_mfma_frac": round(4.0 * pairs * D / t_cap / PEAK_BF16, 4),
+                      "plain_mfma_frac": round(4.0 * pairs * D / t_pl / PEAK_BF16, 4),
+                      "llama_layout_mfma_frac": round(4.0 * pairs * D / t_soft / PEAK_BF16, 4)}
+    seq = torch.arange(nd, dtype=torch.int32, device=dev)
+    cxd = torch.full((nd,), ctx, dtype=torch.int32, device=dev)
+    ws = ops.DecodeWorkspace(nd, H, G, ctx, dev, None, D=D)
+    t_capd = _timed(lambda: ops.softmax_attention_rows(q1[:nd], kr, vr, bt, seq, posd, H, G, D, D, sc, max_ctx=ctx,
+                                                       softcap=30.0, gate=gate[:nd]), iters)
+    t_softd = _timed(lambda: ops.decode_attention(q1[:nd], kr, vt, bt, cxd, H, G, ctx, sc, ws=ws, window=0), iters)
+    kvb = nd * G * ctx * 2 * D * 2.0
+    out["decode"] = {"capped_gated_ms": round(t_capd * 1e3, 4), "llama_layout_ms": round(t_softd * 1e3, 4),
+                     "capped_gated_hbm_frac": round(kvb / t_capd / PEAK_HBM, 4),
+                     "llama_layout_hbm_frac": round(kvb / t_softd / PEAK_HBM, 4)}
+    # ---- experts: T rows (prompts) and nd rows (single tokens)
+    Hd, E, k, F = z["hidden"], u["experts"], u["top"], u["eff"]
+    x = torch.randn(T, Hd, device=dev).to(bf)
+    router = (torch.randn(E, Hd, device=dev) * Hd ** -0.5)
+    corr = torch.randn(E, device=dev) * 0.5 / E
+    w13 = (torch.randn(E, 2 * F, Hd, device=dev) * Hd ** -0.5).to(bf)
+    w2 = (torch.randn(E, Hd, F, device=dev) * F ** -0.5).to(bf)
+    rb = router.to(bf)
+
+    def liz(xx):     # the last two router outputs are identity experts
+        ids, wts = ops.moe_route_grouped(ops.linear(xx.float(), router), corr, k, 4, 2, 2.5)
+        return ops.moe_glu_experts(xx, ids, wts, w13[:E - 2], w2[:E - 2], float("inf"), 1.0, False, shift=0.0, identity=True)
+
+    ex = {}
+    for name, rows in (("prefill", T), ("decode", nd)):
+        xx = x[:rows]
+        fl = 2.0 * rows * k * 3 * Hd * F
+        by = min(E, rows * k) * 3 * Hd * F * 2.0
+        t_l = _timed(lambda: liz(xx), iters)
+        t_m = _timed(lambda: ops.moe_ffn(xx, rb, w13, w2, k), iters)
+        ex[name] = {"lizezen_ms": round(t_l * 1e3, 3), "mixtral_ms": round(t_m * 1e3, 3),
+                    "lizezen_mfma_frac": round(fl / t_l / PEAK_BF16, 4), "mixtral_mfma_frac": round(fl / t_m / PEAK_BF16, 4),
+                    "lizezen_weight_hbm_frac": round(by / t_l / PEAK_HBM, 4),
+                    "mixtral_weight_hbm_frac": round(by / t_m / PEAK_HBM, 4)}
+    out["experts"] = ex
+    del x, w13, w2
+    # ---- row kernels (prompt rows): bytes that must move over the time, against 8 TB/s
+    qkv = torch.randn(T, (H + 2 * G) * D, device=dev).to(bf)
+    slots = torch.arange(T, dtype=torch.int32, device=dev)
+    freq, mag = ops.rotary_frequencies(D, 1e6, (8.0, 4096, 32.0, 1.0))
+    freq = freq.to(dev)
+    hw = torch.ones(D, device=dev)
+    t_rh = _timed(lambda: ops.rope_headnorm_cache_(qkv, posr, slots, kr, vr, H, G, D, D, freq, mag, D, 1e-5, q_w=hw, k_w=hw,
+                                                   v_off=(H + G) * D), iters)
+    cs = ref.rope_cos_sin(L, D, 1e6).to(dev)
+    t_rk = _timed(lambda: ops.rope_cache_(qkv, posr, cs, slots, kr, vt, H, G, D), iters)
+    by_rk = T * (2 * (H + G) * D + 2 * G * D) * 2.0      # q, k read + written, k and v pages written, v read
+    xs = torch.randn(T, Hd, device=dev)
+    y1, y2 = torch.randn(T, Hd, device=dev).to(bf), torch.randn(T, Hd, device=dev).to(bf)
+    wn, bn = torch.ones(Hd, device=dev), torch.zeros(Hd, device=dev)
+    t_rd = _timed(lambda: ops.residual_dyt_(xs, y1, y2, bn, (0.5, wn, bn), bf), iters)
+    xb, wb = xs.to(bf), wn.to(bf)
+    t_an = _timed(lambda: ops.add_rmsnorm(xb, y1, wb, 1e-5), iters)
+    Fd = z["ffn"] // 8 * 8
+    up = torch.randn(T, Fd, device=dev).to(bf)
+    gu = torch.randn(T, 2 * Fd, device=dev).to(bf)
+    bu = torch.randn(Fd, device=dev)
+    t_bg = _timed(lambda: ops.bias_gelu_tanh_(up, bu), iters)
+    t_sm = _timed(lambda: ops.silu_mul(gu), iters)
+    o = torch.randn(T, nv, device=dev)
+    gg = torch.randn(T, nv, device=dev).to(bf)
+    won = torch.ones(nv, device=dev)
+    t_gn = _timed(lambda: ops.group_rmsnorm(o, won, H, 1e-5, bf, gate=gg), iters)
+    out["rows"] = {
+        "rope_headnorm_cache_ms": round(t_rh * 1e3, 3), "rope_headnorm_cache_hbm_frac": round(by_rk / t_rh / PEAK_HBM, 4),
+        "rope_cache_ms": round(t_rk * 1e3, 3), "rope_cache_hbm_frac": round(by_rk / t_rk / PEAK_HBM, 4),
+        "residual_dyt_ms": round(t_rd * 1e3, 3),
+        "residual_dyt_hbm_frac": round(T * Hd * 14.0 / t_rd / PEAK_HBM, 4),      # fp32 in + out, two bf16 in, bf16 out
+        "add_rmsnorm_ms": round(t_an * 1e3, 3), "add_rmsnorm_hbm_frac": round(T * Hd * 8.0 / t_an / PEAK_HBM, 4),
+        "bias_gelu_tanh_ms": round(t_bg * 1e3, 3), "bias_gelu_tanh_hbm_frac": round(T * Fd * 4.0 / t_bg / PEAK_HBM, 4),
+        "silu_mul_ms": round(t_sm * 1e3, 3), "silu_mul_hbm_frac": round(T * Fd * 6.0 / t_sm / PEAK_HBM, 4),
+        "gated_head_norm_ms": round(t_gn * 1e3, 3), "gated_head_norm_hbm_frac": round(T * nv * 8.0 / t_gn / PEAK_HBM, 4)}
+    return out
+
+
 def run(args) -> None:
     names = [s for s in (args.design_sizes or "s,m,l").split(",") if s]
     models = [m for m in (getattr(args, "design_models", None) or "bidasun").split(",") if m]
@@ -379,6 +534,9 @@ def run(args) -> None:
             torch.cuda.empty_cache()
         if "lumepel" in models:
             res[n]["lumepel_kernels"] = lumepel_kernel_times(z)
+            torch.cuda.empty_cache()
+        if "lizezen" in models:
+            res[n]["lizezen_kernels"] = lizezen_kernel_times(z)
             torch.cuda.empty_cache()
         print(f"[designs] {n}: {json.dumps(res[n])}", flush=True)
     line = {"metric": "design_compare", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -1037,7 +1037,7 @@ def lizezen_layers(pattern: Sequence[str], hidden: int, heads: int, kv_heads: in
         elif t in ("attention", "attention_2"):
             second = t == "attention_2"
             rot = RotarySpec(rot_dims or dim, rot_base, False, yarn if second else None)
-            m = RotaryAttentionSpec(heads, heads if second else kv_heads, dim, dim if second else vdim, dim ** -0.5, rot,
+            m = RotaryAttentionSpec(heads, kv_heads, dim, dim if second else vdim, dim ** -0.5, rot,
                                     softcap if second else 0.0, second, second, second)
         else:
             raise ValueError(f"unknown mixer type {t!r}")
