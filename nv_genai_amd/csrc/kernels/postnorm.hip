@@ -267,7 +267,7 @@ template <typename T>
 __global__ void __launch_bounds__(256) group_rmsnorm_kernel(T* __restrict__ out, const float* __restrict__ x,
                                                             const float* __restrict__ w, int64_t n_groups, int gs,
                                                             float eps, int groups, int w_full,
-                                                            const T* __restrict__ gate, int64_t g_stride) {
+                                                            const T* __restrict__ gate, int64_t g_stride, int pair) {
   const int64_t g = blockIdx.x * (int64_t)(blockDim.x >> 6) + (threadIdx.x >> 6);
   if (g >= n_groups) return;
   const int lane = threadIdx.x & 63;
@@ -277,6 +277,25 @@ __global__ void __launch_bounds__(256) group_rmsnorm_kernel(T* __restrict__ out,
   const float* wr = w_full ? w + (int64_t)hg * gs : w;
   const T* gr = gate ? gate + row * g_stride + (int64_t)hg * gs : nullptr;
   float ss = 0.f;
+  if (pair) {   // gs even, 8-byte aligned fp32 rows: two neighbouring elements per lane
+    for (int c = 2 * lane; c < gs; c += 128) {
+      const float2 v = *reinterpret_cast<const float2*>(xr + c);
+      ss += v.x * v.x + v.y * v.y;
+    }
+    ss = wave_sum(ss);
+    const float r = 1.0f / sqrtf(ss / (float)gs + eps);
+    for (int c = 2 * lane; c < gs; c += 128) {
+      const float2 v = *reinterpret_cast<const float2*>(xr + c);
+      float a = v.x * r * wr[c], b = v.y * r * wr[c + 1];
+      if (gr) {
+        a *= 1.0f / (1.0f + expf(-ldf(gr + c)));
+        b *= 1.0f / (1.0f + expf(-ldf(gr + c + 1)));
+      }
+      stf(out + g * gs + c, a);
+      stf(out + g * gs + c + 1, b);
+    }
+    return;
+  }
   for (int c = lane; c < gs; c += 64) ss += xr[c] * xr[c];
   ss = wave_sum(ss);
   const float r = 1.0f / sqrtf(ss / (float)gs + eps);
@@ -317,6 +336,55 @@ __global__ void __launch_bounds__(256) residual_dyt_kernel(float* __restrict__ x
   }
 }
 
+// tanh on the hardware exp2 and reciprocal: for results that are rounded to bf16
+__device__ __forceinline__ float tanh_hw(float x) {
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(2.8853900817779268f * x));
+}
+
+// bf16 rows with H % 4 == 0 and 8-byte aligned rows: 4 elements per thread, 16-byte accesses to
+// the fp32 stream and the fp32 vectors
+__global__ void __launch_bounds__(256) residual_dyt_bf16x4_kernel(float* __restrict__ x, const uint16_t* __restrict__ y1,
+                                                                  int64_t s1, const uint16_t* __restrict__ y2, int64_t s2,
+                                                                  const float* __restrict__ bias, float alpha,
+                                                                  const float* __restrict__ w, const float* __restrict__ b,
+                                                                  uint16_t* __restrict__ out, int64_t T_rows, int H4,
+                                                                  int assign) {
+  const int64_t total = T_rows * H4;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / H4;
+    const int c = (int)(i - r * H4) * 4;
+    const u16x4 a = *reinterpret_cast<const u16x4*>(y1 + r * s1 + c);
+    float y[4] = {bf2f(a[0]), bf2f(a[1]), bf2f(a[2]), bf2f(a[3])};
+    if (y2) {
+      const u16x4 a2 = *reinterpret_cast<const u16x4*>(y2 + r * s2 + c);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) y[j] += bf2f(a2[j]);
+    }
+    if (bias) {
+      const float4 bb = *reinterpret_cast<const float4*>(bias + c);
+      y[0] += bb.x, y[1] += bb.y, y[2] += bb.z, y[3] += bb.w;
+    }
+    float4* xp = reinterpret_cast<float4*>(x + r * 4 * H4 + c);
+    float4 v;
+    if (assign) {
+      v = make_float4(y[0], y[1], y[2], y[3]);
+    } else {
+      v = *xp;
+      v.x += y[0], v.y += y[1], v.z += y[2], v.w += y[3];
+    }
+    *xp = v;
+    if (out) {
+      const float4 ww = *reinterpret_cast<const float4*>(w + c), bn = *reinterpret_cast<const float4*>(b + c);
+      u16x4 o;
+      o[0] = f2bf(tanh_hw(alpha * v.x) * ww.x + bn.x);
+      o[1] = f2bf(tanh_hw(alpha * v.y) * ww.y + bn.y);
+      o[2] = f2bf(tanh_hw(alpha * v.z) * ww.z + bn.z);
+      o[3] = f2bf(tanh_hw(alpha * v.w) * ww.w + bn.w);
+      *reinterpret_cast<u16x4*>(out + r * 4 * H4 + c) = o;
+    }
+  }
+}
+
 // out row = [a row | b row] in the activation type
 template <typename T>
 __global__ void __launch_bounds__(256) pack_pair_kernel(T* __restrict__ out, const float* __restrict__ a,
@@ -340,21 +408,32 @@ __global__ void __launch_bounds__(256) bias_gelu_tanh_kernel(T* __restrict__ x, 
 }
 
 // bf16 rows with F % 8 == 0: 8 elements per thread
+// (a workgroup takes RB whole rows: 32-bit index arithmetic, the bias row stays in cache)
 __global__ void __launch_bounds__(256) bias_gelu_tanh_bf16x8_kernel(uint16_t* __restrict__ x, const float* __restrict__ bias,
-                                                                    int64_t T_rows, int F8) {
-  const int64_t total = T_rows * F8;
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
-    const int c = (int)(i % F8) * 8;
-    const u16x8 v = load8(x + i * 8);
+                                                                    int64_t T_rows, int F8, int RB) {
+  const int64_t r0 = (int64_t)blockIdx.x * RB;
+  const int rows = (int)(T_rows - r0 < RB ? T_rows - r0 : RB);
+  uint16_t* xb = x + r0 * 8 * F8;
+  for (int i = threadIdx.x; i < rows * F8; i += blockDim.x) {
+    const int c = (i % F8) * 8;
+    float bz[8];
+    if (bias) {
+      const float4 b0 = *reinterpret_cast<const float4*>(bias + c), b1 = *reinterpret_cast<const float4*>(bias + c + 4);
+      bz[0] = b0.x, bz[1] = b0.y, bz[2] = b0.z, bz[3] = b0.w, bz[4] = b1.x, bz[5] = b1.y, bz[6] = b1.z, bz[7] = b1.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) bz[j] = 0.f;
+    }
+    const u16x8 v = load8(xb + (int64_t)i * 8);
     u16x8 o;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const float z = bf2f(v[j]) + (bias ? bias[c + j] : 0.f);
+      const float z = bf2f(v[j]) + bz[j];
       const float u = 0.7978845608028654f * (z + 0.044715f * z * z * z);
       // 0.5 z (1 + tanh u) = z - z / (1 + e^(2u))
       o[j] = f2bf(z - z * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(2.8853900817779268f * u)));
     }
-    store8(x + i * 8, o);
+    store8(xb + (int64_t)i * 8, o);
   }
 }
 
@@ -496,12 +575,13 @@ void launch_group_rmsnorm(void* out, const float* x, const float* w, bool w_full
   const int64_t ng = T * groups;
   if (ng == 0) return;
   const unsigned g = (unsigned)((ng + 3) / 4);
+  const int pair = (gs % 2 == 0 && ((uintptr_t)x % 8) == 0) ? 1 : 0;
   if (f32)
     group_rmsnorm_kernel<float><<<dim3(g), 256, 0, stream>>>((float*)out, x, w, ng, gs, eps, groups, w_full ? 1 : 0,
-                                                             (const float*)gate, g_stride);
+                                                             (const float*)gate, g_stride, pair);
   else
     group_rmsnorm_kernel<uint16_t><<<dim3(g), 256, 0, stream>>>((uint16_t*)out, x, w, ng, gs, eps, groups, w_full ? 1 : 0,
-                                                                (const uint16_t*)gate, g_stride);
+                                                                (const uint16_t*)gate, g_stride, pair);
 }
 
 void launch_dyt_norm(void* out, const float* x, float alpha, const float* w, const float* b, const int64_t* rows,
@@ -517,6 +597,16 @@ void launch_residual_dyt(float* x, const void* y1, int64_t s1, const void* y2, i
                          const float* w, const float* b, void* out, int64_t T, int H, bool assign, bool f32,
                          hipStream_t stream) {
   if (T == 0) return;
+  auto al8 = [](const void* p) { return ((uintptr_t)p % 8) == 0; };
+  if (!f32 && H % 4 == 0 && s1 % 4 == 0 && s2 % 4 == 0 && al8(y1) && al8(y2) && al8(out) && ((uintptr_t)x % 16) == 0 &&
+      ((uintptr_t)bias % 16) == 0 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)b % 16) == 0) {
+    int64_t g = (T * (H / 4) + 255) / 256;
+    if (g > 16384) g = 16384;
+    residual_dyt_bf16x4_kernel<<<dim3((unsigned)g), 256, 0, stream>>>(x, (const uint16_t*)y1, s1, (const uint16_t*)y2, s2,
+                                                                      bias, alpha, w, b, (uint16_t*)out, T, H / 4,
+                                                                      assign ? 1 : 0);
+    return;
+  }
   if (f32)
     residual_dyt_kernel<float><<<dim3((unsigned)T), 256, 0, stream>>>(x, (const float*)y1, s1, (const float*)y2, s2, bias,
                                                                      alpha, w, b, (float*)out, H, assign ? 1 : 0);
@@ -536,10 +626,11 @@ void launch_pack_pair(void* out, const float* a, const float* b, int64_t T, int 
 
 void launch_bias_gelu_tanh(void* x, const float* bias, int64_t T, int F, bool f32, hipStream_t stream) {
   if (T == 0 || F == 0) return;
-  if (!f32 && F % 8 == 0 && ((uintptr_t)x % 16) == 0) {
-    int64_t g8 = (T * (F / 8) + 255) / 256;
-    if (g8 > 16384) g8 = 16384;
-    bias_gelu_tanh_bf16x8_kernel<<<dim3((unsigned)g8), 256, 0, stream>>>((uint16_t*)x, bias, T, F / 8);
+  if (!f32 && F % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)bias % 16) == 0) {
+    const int F8 = F / 8;
+    int RB = 2048 / F8;                      // about 8 vectors per thread
+    RB = RB < 1 ? 1 : RB;
+    bias_gelu_tanh_bf16x8_kernel<<<dim3((unsigned)((T + RB - 1) / RB)), 256, 0, stream>>>((uint16_t*)x, bias, T, F8, RB);
     return;
   }
   int64_t g = (T * F + 255) / 256;

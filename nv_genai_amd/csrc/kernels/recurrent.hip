@@ -10,7 +10,9 @@
 //                i = cap tanh((i_pre + b) / cap), f = logsigmoid(cap tanh((f_pre + b) / cap)) and
 //                q scaled by d^(-1/2), all formed in fp32 in the kernel. Same tiling as hgrn2_scan;
 //                the gate chain of a pass (m, both decays, e^(-m)) is run once per pass by one
-//                lane and shared through LDS, the normaliser n is kept beside S in registers.
+//                lane and shared through LDS; the normaliser n is the state of a value column that
+//                is always 1, so every value tile carries it as its last column (VT - 1 value
+//                columns per tile) and n . q comes out of the same partial sums as S^T q.
 //
 // A workgroup owns (segment, head, tile of VT value columns): thread (rg, j) keeps the state
 // elements S[rg * NR + k][j] in registers for the whole segment, so the state is read from its
@@ -214,8 +216,9 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
                                                          const int32_t* __restrict__ cu,
                                                          const int32_t* __restrict__ slots,
                                                          const int32_t* __restrict__ pos, int q_off, int k_off,
-                                                         int v_off, int g_off) {
+                                                         int v_off, int g_off, int vr) {
   constexpr int RG = 256 / VT;
+  constexpr int VR = VT - 1;               // thread column that carries n (a value of 1); value columns: j < vr <= VR
   constexpr int DP = RG * NR;              // padded rows of a head
   constexpr int NQ = TC * DP / 256;        // q (and k) elements a thread stages per pass
   constexpr int NV = (TC * VT + 255) / 256;
@@ -223,7 +226,6 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
   __shared__ __attribute__((aligned(16))) float ks[TC * DP];
   __shared__ float vs[TC * VT];
   __shared__ float part[TC * 256];
-  __shared__ float partn[TC * RG];
   __shared__ float gi[TC], gf[TC];         // log gates of the pass
   __shared__ float ga[TC], gb[TC], gem[TC];   // decay of the old state, weight of the new row, e^(-m)
   __shared__ float m_carry;
@@ -234,22 +236,26 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
   const bool fresh = slot < 0 || pos[t0] == 0;
   const int tid = threadIdx.x;
   const int j = tid % VT, rg = tid / VT;
-  const int col = vt * VT + j;
-  const bool colok = col < dv;
+  const bool is_n = j == VR;               // this thread's column is the normaliser
+  const int col = vt * vr + j;
+  const bool colok = j < vr && col < dv;
   const int64_t ssz = (int64_t)d * dv + d + 1;
   float* sp = slot >= 0 ? state + ((int64_t)slot * H + h) * ssz : nullptr;
-  float S[NR], n[NR];
+  float S[NR];
 #pragma unroll
   for (int k = 0; k < NR; ++k) {
     const int i = rg * NR + k;
-    const bool ld = !fresh && i < d;
-    S[k] = (ld && colok) ? sp[(int64_t)i * dv + col] : 0.f;
-    n[k] = ld ? sp[(int64_t)d * dv + i] : 0.f;
+    float v = 0.f;
+    if (!fresh && i < d) {
+      if (is_n) v = sp[(int64_t)d * dv + i];
+      else if (colok) v = sp[(int64_t)i * dv + col];
+    }
+    S[k] = v;
   }
   if (tid == 0) m_carry = fresh ? 0.f : sp[(int64_t)d * dv + d];
   const float qscale = 1.0f / sqrtf((float)d);
   const float inv_cap = 1.0f / cap;
-  const int qo = q_off + h * d, ko = k_off + h * d, vo = v_off + h * dv + vt * VT;
+  const int qo = q_off + h * d, ko = k_off + h * d, vo = v_off + h * dv + vt * vr;
   float rq[NQ], rk[NQ], rv[NV], ri = 0.f, rf = 0.f;
   // raw values of rows [tc, tc + TC) into registers (rows past t1 and padded columns: zeros)
   auto fetch = [&](int tc) {
@@ -264,7 +270,12 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
 #pragma unroll
     for (int x = 0; x < NV; ++x) {
       const int e = tid + 256 * x, tt = e / VT, jj = e % VT;
-      rv[x] = (e < TC * VT && tc + tt < t1 && vt * VT + jj < dv) ? ldf(proj + (int64_t)(tc + tt) * stride + vo + jj) : 0.f;
+      float v = 0.f;
+      if (e < TC * VT && tc + tt < t1) {
+        if (jj == VR) v = 1.f;
+        else if (jj < vr && vt * vr + jj < dv) v = ldf(proj + (int64_t)(tc + tt) * stride + vo + jj);
+      }
+      rv[x] = v;
     }
     if (tid < TC && tc + tid < t1) {
       const T* pr = proj + (int64_t)(tc + tid) * stride + g_off;
@@ -275,7 +286,7 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
   fetch(t0);
   for (int tc = t0; tc < t1; tc += TC) {
     const int nt = t1 - tc < TC ? t1 - tc : TC;
-    __syncthreads();   // the previous pass is done with the staged rows, part / partn and the gate chain
+    __syncthreads();   // the previous pass is done with the staged rows, part and the gate chain
 #pragma unroll
     for (int x = 0; x < NQ; ++x) {
       const int e = tid + 256 * x;
@@ -292,26 +303,30 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
       gf[tid] = log_sigmoid(cap * tanhf((rf + gate_bias[H + h]) * inv_cap));
     }
     __syncthreads();
-    if (tid == 0) {   // the gate chain of the pass: sequential, a few exponentials per row
-      float m = m_carry;
-      for (int tt = 0; tt < nt; ++tt) {
-        const float fm = gf[tt] + m;
-        const float mn = fmaxf(fm, gi[tt]);
-        ga[tt] = expf(fm - mn);
-        gb[tt] = expf(gi[tt] - mn);
-        gem[tt] = expf(-mn);
-        m = mn;
+    if (tid < TC) {   // the gate chain of the pass: lane t replays the running maximum up to its row
+      // (additions and maxima only, bit-identical to a sequential chain), then the three
+      // exponentials of all rows are taken side by side
+      const float m0 = m_carry;
+      float m = m0, mp = m0;
+      for (int s2 = 0; s2 <= tid && s2 < nt; ++s2) {
+        mp = m;
+        m = fmaxf(gf[s2] + m, gi[s2]);
       }
-      m_carry = m;
+      if (tid < nt) {
+        ga[tid] = expf(gf[tid] + mp - m);
+        gb[tid] = expf(gi[tid] - m);
+        gem[tid] = expf(-m);
+      }
+      if (tid == nt - 1) m_carry = m;
     }
     __syncthreads();
     if (tc + TC < t1) fetch(tc + TC);   // lands while this pass computes
     auto row = [&](int tt) {
       const float a = ga[tt];
-      const float bv = gb[tt] * vs[tt * VT + j], bb = gb[tt];
+      const float bv = gb[tt] * vs[tt * VT + j];
       const float4* kr = reinterpret_cast<const float4*>(ks + tt * DP + rg * NR);
       const float4* qr = reinterpret_cast<const float4*>(qs + tt * DP + rg * NR);
-      float p = 0.f, pn = 0.f;
+      float p = 0.f;
 #pragma unroll
       for (int k4 = 0; k4 < NR / 4; ++k4) {
         const float4 k4v = kr[k4], q4 = qr[k4];
@@ -320,13 +335,10 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
         for (int u = 0; u < 4; ++u) {
           const int k = 4 * k4 + u;
           S[k] = a * S[k] + ka[u] * bv;
-          n[k] = a * n[k] + ka[u] * bb;
           p += S[k] * qa[u];
-          pn += n[k] * qa[u];
         }
       }
       part[tt * 256 + tid] = p;
-      if (j == 0) partn[tt * RG + rg] = pn;
     };
     if (nt == TC) {   // full pass: unrolled, so the LDS reads of later rows run ahead of the recurrence
 #pragma unroll
@@ -335,16 +347,16 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
       for (int tt = 0; tt < nt; ++tt) row(tt);
     }
     __syncthreads();
-    for (int e = tid; e < nt * VT; e += 256) {
-      const int tt = e / VT, jj = e % VT;
-      if (vt * VT + jj < dv) {
+    for (int e = tid; e < nt * vr; e += 256) {
+      const int tt = e / vr, jj = e % vr;
+      if (vt * vr + jj < dv) {
         float s2 = 0.f, nq = 0.f;
 #pragma unroll
         for (int r = 0; r < RG; ++r) {
           s2 += part[tt * 256 + r * VT + jj];
-          nq += partn[tt * RG + r];
+          nq += part[tt * 256 + r * VT + VR];
         }
-        out[(int64_t)(tc + tt) * H * dv + h * dv + vt * VT + jj] = s2 / (fmaxf(fabsf(nq), gem[tt]) + 1e-6f);
+        out[(int64_t)(tc + tt) * H * dv + h * dv + vt * vr + jj] = s2 / (fmaxf(fabsf(nq), gem[tt]) + 1e-6f);
       }
     }
   }
@@ -354,11 +366,10 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
       const int i = rg * NR + k;
       if (i < d) {
         if (colok) sp[(int64_t)i * dv + col] = S[k];
-        if (vt == 0 && j == 0) sp[(int64_t)d * dv + i] = n[k];
+        if (is_n && vt == 0) sp[(int64_t)d * dv + i] = S[k];
       }
     }
-    __syncthreads();   // m_carry of the last pass
-    if (vt == 0 && tid == 0) sp[(int64_t)d * dv + d] = m_carry;
+    if (vt == 0 && tid == 0) sp[(int64_t)d * dv + d] = m_carry;   // of the last pass (a barrier lies in between)
   }
 }
 
@@ -368,11 +379,13 @@ bool launch_mlstm_vt(float* out, const T* proj, int64_t stride, const float* gat
                      int k_off, int v_off, int g_off, hipStream_t stream) {
   constexpr int RG = 256 / VT;
   const int nr = (d + RG - 1) / RG;
-  const dim3 grid((unsigned)((dv + VT - 1) / VT), (unsigned)H, (unsigned)n_seg);
+  const int tiles = (dv + VT - 2) / (VT - 1);
+  const int vr = (dv + tiles - 1) / tiles;   // value columns per tile, balanced over the tiles (<= VT - 1)
+  const dim3 grid((unsigned)tiles, (unsigned)H, (unsigned)n_seg);
 #define NGA_MLSTM_CASE(N)                                                                                            \
   if (nr <= N) {                                                                                                     \
     mlstm_scan_kernel<T, N, VT><<<grid, 256, 0, stream>>>(out, proj, stride, gate_bias, state, H, d, dv, cap, cu, slots, \
-                                                          pos, q_off, k_off, v_off, g_off);                          \
+                                                          pos, q_off, k_off, v_off, g_off, vr);                      \
     return true;                                                                                                     \
   }
   // at most 256 padded rows per head in LDS: NR <= 64 / 32 / 16 for tiles of 64 / 32 / 16 columns
@@ -394,8 +407,8 @@ bool launch_mlstm_t(float* out, const T* proj, int64_t stride, const float* gate
                     float cap, const int32_t* cu, const int32_t* slots, const int32_t* pos, int n_seg, int q_off,
                     int k_off, int v_off, int g_off, hipStream_t stream) {
   const int64_t base = (int64_t)n_seg * H;
-  int vt = dv <= 16 ? 16 : (dv <= 32 ? 32 : 64);
-  while (vt > 16 && base * ((dv + vt - 1) / vt) < 1024) vt /= 2;
+  int vt = dv <= 15 ? 16 : (dv <= 31 ? 32 : 64);   // a tile of vt threads holds vt - 1 value columns and n
+  while (vt > 16 && base * ((dv + vt - 2) / (vt - 1)) < 1024) vt /= 2;
 #define NGA_MLSTM_ARGS out, proj, stride, gate_bias, state, H, d, dv, cap, cu, slots, pos, n_seg, q_off, k_off, v_off, g_off, stream
   if (vt == 64 && launch_mlstm_vt<T, 64>(NGA_MLSTM_ARGS)) return true;
   if (vt >= 32 && launch_mlstm_vt<T, 32>(NGA_MLSTM_ARGS)) return true;

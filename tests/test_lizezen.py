@@ -202,19 +202,22 @@ def test_rotary_frequencies_against_the_oracle():
         assert torch.allclose(f, fo, rtol=1e-14, atol=0) and abs(mag - mo) < 1e-15
 
 
+@pytest.mark.parametrize("sizes", [(4, 2, 10, 6, 7, 3), (5, 2, 32, 32, 16, 8), (3, 3, 128, 128, 64, 0), (9, 1, 16, 16, 8, 8)])
 @pytest.mark.parametrize("from_keys", [False, True])
 @pytest.mark.parametrize("device,dtype", DTYPES)
-def test_head_norm_rotation_and_page_write(device, dtype, from_keys):
-    """Positions far out (the angle must stay exact), a rotation on part of the head, slots in
-    several pages, a row that is not written; values from their own columns or from the keys as
-    projected (before norm and rotation)."""
+def test_head_norm_rotation_and_page_write(device, dtype, from_keys, sizes):
+    """Positions far out (the angle must stay exact), a rotation on part of the head or on all of
+    it (sizes the 16-byte form takes, more heads than one round of a wave holds), slots in several
+    pages, a row that is not written; values from their own columns or from the keys as projected
+    (before norm and rotation)."""
     tdt = tdtype(dtype)
     g = torch.Generator().manual_seed(5)
-    T, H, G, dk, dims = 9, 4, 2, 10, 6
-    dv = dk if from_keys else 7
+    H, G, dk, dims, dv, pad = sizes
+    T = 9
+    dv = dk if from_keys else dv
     rot = {"dims": dims, "base": 30.0, "scaling": {"factor": 4.0, "original": 16, "fast": 4.0, "slow": 1.0}}
     freq, mag = ops.rotary_frequencies(dims, 30.0, (4.0, 16, 4.0, 1.0))
-    cols = (H + G) * dk + (0 if from_keys else G * dv) + 3
+    cols = (H + G) * dk + (0 if from_keys else G * dv) + pad
     proj0 = torch.randn(T, cols, generator=g).to(tdt)
     pos = torch.tensor([0, 1, 63, 64, 1000, 65535, 99999, 7, 2], dtype=torch.int32)
     slots = torch.tensor([0, 1, 63, 64, 130, 191, 5, -1, 70], dtype=torch.int32)
