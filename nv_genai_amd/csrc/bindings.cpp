@@ -1497,8 +1497,8 @@ void mlstm_scan(Tensor out, Tensor proj, Tensor gate_bias, Tensor state, int64_t
               v_off + H * dv <= W && g_off + 2 * H <= W, "mlstm_scan: columns outside the rows");
   TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == H * dv && pos.numel() == T);
   TORCH_CHECK(gate_bias.numel() == 2 * H);
-  TORCH_CHECK(state.dim() == 3 && state.size(1) == H && state.size(2) == d * dv + d + 1,
-              "mlstm_scan: state must be [slots, H, d * dv + d + 1]");
+  TORCH_CHECK(state.dim() == 3 && state.size(1) == H && state.size(2) == d * dv + (dv + 15) / 16 * (d + 1),
+              "mlstm_scan: state must be [slots, H, d * dv + ceil(dv / 16) * (d + 1)]");
   TORCH_CHECK(d <= nga::mlstm_max_dim(), "mlstm_scan: the per-head key size exceeds the kernel's register tile");
   const int n = (int)slots.numel();
   const int32_t* cp = nullptr;

@@ -375,7 +375,7 @@ void launch_softmax_decode_mfma(uint16_t* out, float* ws, int parts, const uint1
 
 // recurrent.hip
 int mlstm_max_dim();
-// state [slots, H, d * dv + d + 1] fp32 (S, n, m); gate columns [i (H) | f (H)] from g_off
+// state [slots, H, d * dv + ceil(dv / 16) * (d + 1)] fp32 (S, then copies of (n, m)); gate columns [i (H) | f (H)] from g_off
 bool launch_mlstm_scan(float* out, const void* proj, int64_t stride, const float* gate_bias, float* state, int H, int d,
                        int dv, float cap, const int32_t* cu, const int32_t* slots, const int32_t* pos, int n_seg,
                        int q_off, int k_off, int v_off, int g_off, bool f32, hipStream_t stream);

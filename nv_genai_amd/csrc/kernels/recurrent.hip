@@ -9,10 +9,11 @@
 //                o = S^T q / (max(|n . q|, e^(-m')) + 1e-6), with the log gates
 //                i = cap tanh((i_pre + b) / cap), f = logsigmoid(cap tanh((f_pre + b) / cap)) and
 //                q scaled by d^(-1/2), all formed in fp32 in the kernel. Same tiling as hgrn2_scan;
-//                the gate chain of a pass (m, both decays, e^(-m)) is run once per pass by one
-//                lane and shared through LDS; the normaliser n is the state of a value column that
-//                is always 1, so every value tile carries it as its last column (VT - 1 value
-//                columns per tile) and n . q comes out of the same partial sums as S^T q.
+//                every value tile carries n and m itself (they do not depend on the value column)
+//                and the state slot keeps one copy of (n, m) per 16 value columns: a tile reads the
+//                copy of its first columns and writes the copies of its own columns, so no tile
+//                reads what another tile of the launch writes. The gate chain of a pass (m, both
+//                decays, e^(-m)) is a prefix scan over the lanes of the first wave, shared through LDS.
 //
 // A workgroup owns (segment, head, tile of VT value columns): thread (rg, j) keeps the state
 // elements S[rg * NR + k][j] in registers for the whole segment, so the state is read from its
@@ -205,7 +206,7 @@ bool launch_hgrn2_t(float* out, const T* proj, int64_t stride, const float* f_bi
 
 // ---------------------------------------------------------------------------------------------
 // mLSTM. proj row: q [H*d] at q_off, k [H*d] at k_off, v [H*dv] at v_off, gate pre-activations
-// [i (H) | f (H)] at g_off. State slot of a head: S [d][dv], n [d], m (d * dv + d + 1 floats).
+// [i (H) | f (H)] at g_off. State slot of a head: S [d][dv], then ceil(dv / 16) copies of (n [d], m).
 // cu == nullptr: segment b is row b. Padded state rows (i >= d) see k = q = 0 and stay 0.
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
@@ -216,9 +217,8 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
                                                          const int32_t* __restrict__ cu,
                                                          const int32_t* __restrict__ slots,
                                                          const int32_t* __restrict__ pos, int q_off, int k_off,
-                                                         int v_off, int g_off, int vr) {
+                                                         int v_off, int g_off) {
   constexpr int RG = 256 / VT;
-  constexpr int VR = VT - 1;               // thread column that carries n (a value of 1); value columns: j < vr <= VR
   constexpr int DP = RG * NR;              // padded rows of a head
   constexpr int NQ = TC * DP / 256;        // q (and k) elements a thread stages per pass
   constexpr int NV = (TC * VT + 255) / 256;
@@ -226,6 +226,7 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
   __shared__ __attribute__((aligned(16))) float ks[TC * DP];
   __shared__ float vs[TC * VT];
   __shared__ float part[TC * 256];
+  __shared__ float partn[TC * RG];
   __shared__ float gi[TC], gf[TC];         // log gates of the pass
   __shared__ float ga[TC], gb[TC], gem[TC];   // decay of the old state, weight of the new row, e^(-m)
   __shared__ float m_carry;
@@ -236,26 +237,27 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
   const bool fresh = slot < 0 || pos[t0] == 0;
   const int tid = threadIdx.x;
   const int j = tid % VT, rg = tid / VT;
-  const bool is_n = j == VR;               // this thread's column is the normaliser
-  const int col = vt * vr + j;
-  const bool colok = j < vr && col < dv;
-  const int64_t ssz = (int64_t)d * dv + d + 1;
+  const int col = vt * VT + j;
+  const bool colok = col < dv;
+  const int ncopy = (dv + 15) / 16;        // copies of (n, m): one per 16 value columns
+  const int64_t ssz = (int64_t)d * dv + (int64_t)ncopy * (d + 1);
   float* sp = slot >= 0 ? state + ((int64_t)slot * H + h) * ssz : nullptr;
-  float S[NR];
+  // this tile reads the copy of its first 16 columns and writes the copies of all its columns: no
+  // tile reads what another tile of the launch writes, whatever tile widths the launches use
+  const int c0 = vt * (VT / 16), c1 = min(ncopy, (vt + 1) * (VT / 16));
+  const float* nm_in = sp ? sp + (int64_t)d * dv + (int64_t)c0 * (d + 1) : nullptr;
+  float S[NR], n[NR];
 #pragma unroll
   for (int k = 0; k < NR; ++k) {
     const int i = rg * NR + k;
-    float v = 0.f;
-    if (!fresh && i < d) {
-      if (is_n) v = sp[(int64_t)d * dv + i];
-      else if (colok) v = sp[(int64_t)i * dv + col];
-    }
-    S[k] = v;
+    const bool ld = !fresh && i < d;
+    S[k] = (ld && colok) ? sp[(int64_t)i * dv + col] : 0.f;
+    n[k] = ld ? nm_in[i] : 0.f;
   }
-  if (tid == 0) m_carry = fresh ? 0.f : sp[(int64_t)d * dv + d];
+  if (tid == 0) m_carry = fresh ? 0.f : nm_in[d];
   const float qscale = 1.0f / sqrtf((float)d);
   const float inv_cap = 1.0f / cap;
-  const int qo = q_off + h * d, ko = k_off + h * d, vo = v_off + h * dv + vt * vr;
+  const int qo = q_off + h * d, ko = k_off + h * d, vo = v_off + h * dv + vt * VT;
   float rq[NQ], rk[NQ], rv[NV], ri = 0.f, rf = 0.f;
   // raw values of rows [tc, tc + TC) into registers (rows past t1 and padded columns: zeros)
   auto fetch = [&](int tc) {
@@ -270,12 +272,7 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
 #pragma unroll
     for (int x = 0; x < NV; ++x) {
       const int e = tid + 256 * x, tt = e / VT, jj = e % VT;
-      float v = 0.f;
-      if (e < TC * VT && tc + tt < t1) {
-        if (jj == VR) v = 1.f;
-        else if (jj < vr && vt * vr + jj < dv) v = ldf(proj + (int64_t)(tc + tt) * stride + vo + jj);
-      }
-      rv[x] = v;
+      rv[x] = (e < TC * VT && tc + tt < t1 && vt * VT + jj < dv) ? ldf(proj + (int64_t)(tc + tt) * stride + vo + jj) : 0.f;
     }
     if (tid < TC && tc + tid < t1) {
       const T* pr = proj + (int64_t)(tc + tid) * stride + g_off;
@@ -286,7 +283,7 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
   fetch(t0);
   for (int tc = t0; tc < t1; tc += TC) {
     const int nt = t1 - tc < TC ? t1 - tc : TC;
-    __syncthreads();   // the previous pass is done with the staged rows, part and the gate chain
+    __syncthreads();   // the previous pass is done with the staged rows, part / partn and the gate chain
 #pragma unroll
     for (int x = 0; x < NQ; ++x) {
       const int e = tid + 256 * x;
@@ -303,30 +300,43 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
       gf[tid] = log_sigmoid(cap * tanhf((rf + gate_bias[H + h]) * inv_cap));
     }
     __syncthreads();
-    if (tid < TC) {   // the gate chain of the pass: lane t replays the running maximum up to its row
-      // (additions and maxima only, bit-identical to a sequential chain), then the three
-      // exponentials of all rows are taken side by side
-      const float m0 = m_carry;
-      float m = m0, mp = m0;
-      for (int s2 = 0; s2 <= tid && s2 < nt; ++s2) {
-        mp = m;
-        m = fmaxf(gf[s2] + m, gi[s2]);
-      }
+    if (tid < 64) {   // the gate chain of the pass on the first wave, one row per lane: the running
+      // maximum m_t = max(f_t + m_(t-1), i_t) is a prefix scan over the maps m -> max(m + A, B),
+      // composed as (A1, B1) then (A2, B2) = (A1 + A2, max(B1 + A2, B2)); lanes past the pass's
+      // rows hold the identity. The three exponentials of all rows are then taken side by side.
+      float A = 0.f, B = -INFINITY;
       if (tid < nt) {
-        ga[tid] = expf(gf[tid] + mp - m);
-        gb[tid] = expf(gi[tid] - m);
+        A = gf[tid];
+        B = gi[tid];
+      }
+      const float f_t = A, i_t = B;
+#pragma unroll
+      for (int o = 1; o < TC; o <<= 1) {
+        const float Ap = __shfl_up(A, o, 64), Bp = __shfl_up(B, o, 64);
+        if (tid >= o) {
+          B = fmaxf(Bp + A, B);
+          A = Ap + A;
+        }
+      }
+      const float m0 = m_carry;
+      const float m = fmaxf(m0 + A, B);
+      float mp = __shfl_up(m, 1, 64);
+      if (tid == 0) mp = m0;
+      if (tid < nt) {
+        ga[tid] = expf(f_t + mp - m);
+        gb[tid] = expf(i_t - m);
         gem[tid] = expf(-m);
       }
-      if (tid == nt - 1) m_carry = m;
+      if (tid == TC - 1) m_carry = m;      // (lanes past nt pass the last row's maximum on)
     }
     __syncthreads();
     if (tc + TC < t1) fetch(tc + TC);   // lands while this pass computes
     auto row = [&](int tt) {
       const float a = ga[tt];
-      const float bv = gb[tt] * vs[tt * VT + j];
+      const float bv = gb[tt] * vs[tt * VT + j], bb = gb[tt];
       const float4* kr = reinterpret_cast<const float4*>(ks + tt * DP + rg * NR);
       const float4* qr = reinterpret_cast<const float4*>(qs + tt * DP + rg * NR);
-      float p = 0.f;
+      float p = 0.f, pn = 0.f;
 #pragma unroll
       for (int k4 = 0; k4 < NR / 4; ++k4) {
         const float4 k4v = kr[k4], q4 = qr[k4];
@@ -335,10 +345,13 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
         for (int u = 0; u < 4; ++u) {
           const int k = 4 * k4 + u;
           S[k] = a * S[k] + ka[u] * bv;
+          n[k] = a * n[k] + ka[u] * bb;
           p += S[k] * qa[u];
+          pn += n[k] * qa[u];
         }
       }
       part[tt * 256 + tid] = p;
+      if (j == 0) partn[tt * RG + rg] = pn;
     };
     if (nt == TC) {   // full pass: unrolled, so the LDS reads of later rows run ahead of the recurrence
 #pragma unroll
@@ -347,29 +360,30 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
       for (int tt = 0; tt < nt; ++tt) row(tt);
     }
     __syncthreads();
-    for (int e = tid; e < nt * vr; e += 256) {
-      const int tt = e / vr, jj = e % vr;
-      if (vt * vr + jj < dv) {
+    for (int e = tid; e < nt * VT; e += 256) {
+      const int tt = e / VT, jj = e % VT;
+      if (vt * VT + jj < dv) {
         float s2 = 0.f, nq = 0.f;
 #pragma unroll
         for (int r = 0; r < RG; ++r) {
           s2 += part[tt * 256 + r * VT + jj];
-          nq += part[tt * 256 + r * VT + VR];
+          nq += partn[tt * RG + r];
         }
-        out[(int64_t)(tc + tt) * H * dv + h * dv + vt * vr + jj] = s2 / (fmaxf(fabsf(nq), gem[tt]) + 1e-6f);
+        out[(int64_t)(tc + tt) * H * dv + h * dv + vt * VT + jj] = s2 / (fmaxf(fabsf(nq), gem[tt]) + 1e-6f);
       }
     }
   }
   if (sp) {
+    __syncthreads();   // m_carry of the last pass
 #pragma unroll
     for (int k = 0; k < NR; ++k) {
       const int i = rg * NR + k;
       if (i < d) {
         if (colok) sp[(int64_t)i * dv + col] = S[k];
-        if (is_n && vt == 0) sp[(int64_t)d * dv + i] = S[k];
+        if (j < c1 - c0) sp[(int64_t)d * dv + (int64_t)(c0 + j) * (d + 1) + i] = n[k];   // thread j: copy c0 + j
       }
     }
-    if (vt == 0 && tid == 0) sp[(int64_t)d * dv + d] = m_carry;   // of the last pass (a barrier lies in between)
+    if (tid < c1 - c0) sp[(int64_t)d * dv + (int64_t)(c0 + tid) * (d + 1) + d] = m_carry;
   }
 }
 
@@ -379,13 +393,11 @@ bool launch_mlstm_vt(float* out, const T* proj, int64_t stride, const float* gat
                      int k_off, int v_off, int g_off, hipStream_t stream) {
   constexpr int RG = 256 / VT;
   const int nr = (d + RG - 1) / RG;
-  const int tiles = (dv + VT - 2) / (VT - 1);
-  const int vr = (dv + tiles - 1) / tiles;   // value columns per tile, balanced over the tiles (<= VT - 1)
-  const dim3 grid((unsigned)tiles, (unsigned)H, (unsigned)n_seg);
+  const dim3 grid((unsigned)((dv + VT - 1) / VT), (unsigned)H, (unsigned)n_seg);
 #define NGA_MLSTM_CASE(N)                                                                                            \
   if (nr <= N) {                                                                                                     \
     mlstm_scan_kernel<T, N, VT><<<grid, 256, 0, stream>>>(out, proj, stride, gate_bias, state, H, d, dv, cap, cu, slots, \
-                                                          pos, q_off, k_off, v_off, g_off, vr);                      \
+                                                          pos, q_off, k_off, v_off, g_off);                          \
     return true;                                                                                                     \
   }
   // at most 256 padded rows per head in LDS: NR <= 64 / 32 / 16 for tiles of 64 / 32 / 16 columns
@@ -407,8 +419,8 @@ bool launch_mlstm_t(float* out, const T* proj, int64_t stride, const float* gate
                     float cap, const int32_t* cu, const int32_t* slots, const int32_t* pos, int n_seg, int q_off,
                     int k_off, int v_off, int g_off, hipStream_t stream) {
   const int64_t base = (int64_t)n_seg * H;
-  int vt = dv <= 15 ? 16 : (dv <= 31 ? 32 : 64);   // a tile of vt threads holds vt - 1 value columns and n
-  while (vt > 16 && base * ((dv + vt - 2) / (vt - 1)) < 1024) vt /= 2;
+  int vt = dv <= 16 ? 16 : (dv <= 32 ? 32 : 64);
+  while (vt > 16 && base * ((dv + vt - 1) / vt) < 1024) vt /= 2;
 #define NGA_MLSTM_ARGS out, proj, stride, gate_bias, state, H, d, dv, cap, cu, slots, pos, n_seg, q_off, k_off, v_off, g_off, stream
   if (vt == 64 && launch_mlstm_vt<T, 64>(NGA_MLSTM_ARGS)) return true;
   if (vt >= 32 && launch_mlstm_vt<T, 32>(NGA_MLSTM_ARGS)) return true;

@@ -235,7 +235,7 @@ class LizezenModel:
         return self.k_cache, self.v_cache
 
     def allocate_state(self, slots: int) -> None:
-        """Recurrent state: per run of an ``mlstm`` layer fp32 [slots, heads, dim * vdim + dim + 1]
+        """Recurrent state: per run of an ``mlstm`` layer fp32 [slots, heads, ops.mlstm_state_size]
         (S, n, m of every head). A slot needs no clearing when it is given to a new sequence: a
         segment that starts at position 0 starts from zeros, not from the slot."""
         self.rec_state = []

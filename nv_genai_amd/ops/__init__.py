@@ -808,8 +808,10 @@ def hgrn2_scan(proj, f_bias, lower, state, H: int, d: int, dv: int, cu, slots, p
 
 
 def mlstm_state_size(d: int, dv: int) -> int:
-    """fp32 elements of one head's mLSTM state: S [d, dv], n [d], m."""
-    return d * dv + d + 1
+    """fp32 elements of one head's mLSTM state: S [d, dv], then one copy of (n [d], m) per 16
+    value columns (every value tile of the scan kernel keeps the copies of its own columns, so
+    no tile reads what another writes; all copies hold the same numbers)."""
+    return d * dv + -(-dv // 16) * (d + 1)
 
 
 def mlstm_scan(proj, gate_bias, state, H: int, d: int, dv: int, cap: float, cu, slots, pos, offs) -> torch.Tensor:
@@ -821,7 +823,7 @@ def mlstm_scan(proj, gate_bias, state, H: int, d: int, dv: int, cap: float, cu, 
     ``S <- e^(f + m - m') S + e^(i - m') k v^T``, ``n`` likewise with k alone,
     ``o = S^T q / (max(|n . q|, e^(-m')) + 1e-6)``. Segment b is rows ``cu[b] .. cu[b + 1]``
     (``cu`` None: row b alone) of one sequence; its state (S, n, m) comes from ``state[slots[b]]``
-    ([slots, H, d * dv + d + 1] fp32), or zeros (m = 0) when the segment starts at position 0 - a
+    ([slots, H, mlstm_state_size(d, dv)] fp32), or zeros (m = 0) when the segment starts at position 0 - a
     reused slot needs no clearing - and goes back there. ``slots[b]`` < 0: nothing is read or
     kept. Returns the fp32 outputs [T, H*dv]."""
     if not _gpu(proj):

@@ -859,8 +859,9 @@ def mlstm_scan(proj, gate_bias, state, H, d, dv, cap, cu, slots, pos, offs):
             m = m_new
             den = torch.maximum((nn * q[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
             out[t] = torch.einsum("hdv,hd->hv", S, q[t]) / den[:, None]
-        if sl >= 0:
-            state[sl] = torch.cat([S.reshape(H, d * dv), nn, m[:, None]], dim=1)
+        if sl >= 0:   # S, then the copies of (n, m) the kernel's layout holds (one per 16 value columns)
+            nm = torch.cat([nn, m[:, None]], dim=1)
+            state[sl] = torch.cat([S.reshape(H, d * dv)] + [nm] * (-(-dv // 16)), dim=1)
     return out.reshape(T, H * dv)
 
 
