@@ -496,7 +496,7 @@ def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--llm", default="llama3-8b",
                     help="LLM preset, or a model folder (config.json + safetensors: the design named there, "
-                         "e.g. Bidasun, Biruvik or Lumepel, picks the model class); '' to disable")
+                         "e.g. Bidasun, Biruvik, Lumepel or Lizezen, picks the model class); '' to disable")
     ap.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"), help="LLM dtype")
     ap.add_argument("--embed", default="arctic-embed-l", help="encoder preset ('' to disable)")
     ap.add_argument("--rerank", default="", help="reranker preset ('' to disable)")
