@@ -943,15 +943,14 @@ class LizezenConfig:
             elif t in ("attention", "attention_2"):
                 second = t == "attention_2"
                 dim = int(m["dim"])
+                # (values that are the keys have the keys' size, whatever the config says about vdim)
                 mixer = RotaryAttentionSpec(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=dim,
-                                            vdim=int(m.get("vdim", dim)), scale=float(m["scale"]),
+                                            vdim=dim if second else int(m.get("vdim", dim)), scale=float(m["scale"]),
                                             rot=cls._rot(m["rot"], f"layer {i}", dim),
                                             softcap=float(m.get("softcap") or 0.0), qk_norm=second,
                                             values_from_keys=second, head_gate=second)
                 if mixer.heads % mixer.kv_heads:
                     raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
-                if second and mixer.vdim != mixer.dim:
-                    raise ValueError(f"layer {i}: values taken from the keys need vdim = dim")
             else:
                 raise ValueError(f"layer {i}: unknown mixer type {t!r} (known: {_LIZEZEN_MIXERS})")
             if min(mixer.heads, mixer.dim, mixer.vdim) < 1:
