@@ -51,7 +51,7 @@ def _engine(kind: str, z: dict, max_len: int, pages: int, seqs: int):
         mcfg = lizezen_layers(pat, z["hidden"], z["heads"], z["kv"], z["d"], z["d"], z["ffn"], mlstm_heads=z["heads"],
                               mlstm_dim=LIZEZEN_MLSTM["dim"], mlstm_vdim=LIZEZEN_MLSTM["vdim"], experts=u["experts"] - 2,
                               top=u["top"], expert_ff=u["eff"], shared_ff=u["eff"], identity=2, groups=4, keep=2,
-                              route_scale=2.5, softcap=30.0, rot_base=1e6, yarn=(8.0, 4096, 32.0, 1.0), vocab_size=VOCAB)
+                              route_scale=2.0, softcap=30.0, rot_base=1e6, yarn=(8.0, 4096, 32.0, 1.0), vocab_size=VOCAB)
     elif kind == "lumepel":
         u = z["lumepel"]
         pat = [LUMEPEL_PATTERN[i % len(LUMEPEL_PATTERN)] for i in range(z["layers"])]
@@ -459,7 +459,7 @@ def lizezen_kernel_times(z: dict, iters: int = 20) -> dict:
     rb = router.to(bf)
 
     def liz(xx):     # the last two router outputs are identity experts
-        ids, wts = ops.moe_route_grouped(ops.linear(xx.float(), router), corr, k, 4, 2, 2.5)
+        ids, wts = ops.moe_route_grouped(ops.linear(xx.float(), router), corr, k, 4, 2, 2.0)
         return ops.moe_glu_experts(xx, ids, wts, w13[:E - 2], w2[:E - 2], float("inf"), 1.0, False, shift=0.0, identity=True)
 
     ex = {}
