@@ -210,7 +210,9 @@ bool launch_hgrn2_t(float* out, const T* proj, int64_t stride, const float* f_bi
 // cu == nullptr: segment b is row b. Padded state rows (i >= d) see k = q = 0 and stay 0.
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
-template <typename T, int NR, int VT>
+// TCN: rows staged per pass (16 for prompt portions; 1 for launches whose segments are single rows: a
+// sixteenth of the LDS, so that all workgroups of a decode step are resident at once)
+template <typename T, int NR, int VT, int TCN>
 __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out, const T* __restrict__ proj,
                                                          int64_t stride, const float* __restrict__ gate_bias,
                                                          float* __restrict__ state, int H, int d, int dv, float cap,
@@ -220,15 +222,15 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
                                                          int v_off, int g_off) {
   constexpr int RG = 256 / VT;
   constexpr int DP = RG * NR;              // padded rows of a head
-  constexpr int NQ = TC * DP / 256;        // q (and k) elements a thread stages per pass
-  constexpr int NV = (TC * VT + 255) / 256;
-  __shared__ __attribute__((aligned(16))) float qs[TC * DP];
-  __shared__ __attribute__((aligned(16))) float ks[TC * DP];
-  __shared__ float vs[TC * VT];
-  __shared__ float part[TC * 256];
-  __shared__ float partn[TC * RG];
-  __shared__ float gi[TC], gf[TC];         // log gates of the pass
-  __shared__ float ga[TC], gb[TC], gem[TC];   // decay of the old state, weight of the new row, e^(-m)
+  constexpr int NQ = (TCN * DP + 255) / 256;   // q (and k) elements a thread stages per pass
+  constexpr int NV = (TCN * VT + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float qs[TCN * DP];
+  __shared__ __attribute__((aligned(16))) float ks[TCN * DP];
+  __shared__ float vs[TCN * VT];
+  __shared__ float part[TCN * 256];
+  __shared__ float partn[TCN * RG];
+  __shared__ float gi[TCN], gf[TCN];         // log gates of the pass
+  __shared__ float ga[TCN], gb[TCN], gem[TCN];   // decay of the old state, weight of the new row, e^(-m)
   __shared__ float m_carry;
   const int vt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int t0 = cu ? cu[b] : b, t1 = cu ? cu[b + 1] : b + 1;
@@ -247,24 +249,27 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
   const int c0 = vt * (VT / 16), c1 = min(ncopy, (vt + 1) * (VT / 16));
   const float* nm_in = sp ? sp + (int64_t)d * dv + (int64_t)c0 * (d + 1) : nullptr;
   float S[NR], n[NR];
+  // n goes through LDS: one global access per element and workgroup instead of one per thread
+  if (!fresh && tid < d) part[tid] = nm_in[tid];
+  __syncthreads();
 #pragma unroll
   for (int k = 0; k < NR; ++k) {
     const int i = rg * NR + k;
     const bool ld = !fresh && i < d;
     S[k] = (ld && colok) ? sp[(int64_t)i * dv + col] : 0.f;
-    n[k] = ld ? nm_in[i] : 0.f;
+    n[k] = ld ? part[i] : 0.f;
   }
   if (tid == 0) m_carry = fresh ? 0.f : nm_in[d];
   const float qscale = 1.0f / sqrtf((float)d);
   const float inv_cap = 1.0f / cap;
   const int qo = q_off + h * d, ko = k_off + h * d, vo = v_off + h * dv + vt * VT;
   float rq[NQ], rk[NQ], rv[NV], ri = 0.f, rf = 0.f;
-  // raw values of rows [tc, tc + TC) into registers (rows past t1 and padded columns: zeros)
+  // raw values of rows [tc, tc + TCN) into registers (rows past t1 and padded columns: zeros)
   auto fetch = [&](int tc) {
 #pragma unroll
     for (int x = 0; x < NQ; ++x) {
       const int e = tid + 256 * x, tt = e / DP, i = e % DP;
-      const bool ok = tc + tt < t1 && i < d;
+      const bool ok = e < TCN * DP && tc + tt < t1 && i < d;
       const T* pr = proj + (int64_t)(tc + tt) * stride;
       rq[x] = ok ? ldf(pr + qo + i) : 0.f;
       rk[x] = ok ? ldf(pr + ko + i) : 0.f;
@@ -272,30 +277,32 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
 #pragma unroll
     for (int x = 0; x < NV; ++x) {
       const int e = tid + 256 * x, tt = e / VT, jj = e % VT;
-      rv[x] = (e < TC * VT && tc + tt < t1 && vt * VT + jj < dv) ? ldf(proj + (int64_t)(tc + tt) * stride + vo + jj) : 0.f;
+      rv[x] = (e < TCN * VT && tc + tt < t1 && vt * VT + jj < dv) ? ldf(proj + (int64_t)(tc + tt) * stride + vo + jj) : 0.f;
     }
-    if (tid < TC && tc + tid < t1) {
+    if (tid < TCN && tc + tid < t1) {
       const T* pr = proj + (int64_t)(tc + tid) * stride + g_off;
       ri = ldf(pr + h);
       rf = ldf(pr + H + h);
     }
   };
   fetch(t0);
-  for (int tc = t0; tc < t1; tc += TC) {
-    const int nt = t1 - tc < TC ? t1 - tc : TC;
+  for (int tc = t0; tc < t1; tc += TCN) {
+    const int nt = t1 - tc < TCN ? t1 - tc : TCN;
     __syncthreads();   // the previous pass is done with the staged rows, part / partn and the gate chain
 #pragma unroll
     for (int x = 0; x < NQ; ++x) {
       const int e = tid + 256 * x;
-      qs[e] = rq[x] * qscale;
-      ks[e] = rk[x];
+      if (e < TCN * DP) {
+        qs[e] = rq[x] * qscale;
+        ks[e] = rk[x];
+      }
     }
 #pragma unroll
     for (int x = 0; x < NV; ++x) {
       const int e = tid + 256 * x;
-      if (e < TC * VT) vs[e] = rv[x];
+      if (e < TCN * VT) vs[e] = rv[x];
     }
-    if (tid < TC) {
+    if (tid < TCN) {
       gi[tid] = cap * tanhf((ri + gate_bias[h]) * inv_cap);
       gf[tid] = log_sigmoid(cap * tanhf((rf + gate_bias[H + h]) * inv_cap));
     }
@@ -311,7 +318,7 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
       }
       const float f_t = A, i_t = B;
 #pragma unroll
-      for (int o = 1; o < TC; o <<= 1) {
+      for (int o = 1; o < TCN; o <<= 1) {
         const float Ap = __shfl_up(A, o, 64), Bp = __shfl_up(B, o, 64);
         if (tid >= o) {
           B = fmaxf(Bp + A, B);
@@ -327,10 +334,10 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
         gb[tid] = expf(i_t - m);
         gem[tid] = expf(-m);
       }
-      if (tid == TC - 1) m_carry = m;      // (lanes past nt pass the last row's maximum on)
+      if (tid == TCN - 1) m_carry = m;      // (lanes past nt pass the last row's maximum on)
     }
     __syncthreads();
-    if (tc + TC < t1) fetch(tc + TC);   // lands while this pass computes
+    if (tc + TCN < t1) fetch(tc + TCN);   // lands while this pass computes
     auto row = [&](int tt) {
       const float a = ga[tt];
       const float bv = gb[tt] * vs[tt * VT + j], bb = gb[tt];
@@ -353,9 +360,9 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
       part[tt * 256 + tid] = p;
       if (j == 0) partn[tt * RG + rg] = pn;
     };
-    if (nt == TC) {   // full pass: unrolled, so the LDS reads of later rows run ahead of the recurrence
+    if (nt == TCN) {   // full pass: unrolled, so the LDS reads of later rows run ahead of the recurrence
 #pragma unroll
-      for (int tt = 0; tt < TC; ++tt) row(tt);
+      for (int tt = 0; tt < TCN; ++tt) row(tt);
     } else {
       for (int tt = 0; tt < nt; ++tt) row(tt);
     }
@@ -374,20 +381,23 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
     }
   }
   if (sp) {
-    __syncthreads();   // m_carry of the last pass
+    __syncthreads();   // m_carry of the last pass; the last pass is done with part
 #pragma unroll
     for (int k = 0; k < NR; ++k) {
       const int i = rg * NR + k;
-      if (i < d) {
-        if (colok) sp[(int64_t)i * dv + col] = S[k];
-        if (j < c1 - c0) sp[(int64_t)d * dv + (int64_t)(c0 + j) * (d + 1) + i] = n[k];   // thread j: copy c0 + j
-      }
+      if (i < d && colok) sp[(int64_t)i * dv + col] = S[k];
+      if (j == 0) part[i] = n[k];
+    }
+    __syncthreads();
+    for (int e = tid; e < (c1 - c0) * d; e += 256) {   // the copies of n this tile owns
+      const int c = e / d, i = e - c * d;
+      sp[(int64_t)d * dv + (int64_t)(c0 + c) * (d + 1) + i] = part[i];
     }
     if (tid < c1 - c0) sp[(int64_t)d * dv + (int64_t)(c0 + tid) * (d + 1) + d] = m_carry;
   }
 }
 
-template <typename T, int VT>
+template <typename T, int VT, int TCN>
 bool launch_mlstm_vt(float* out, const T* proj, int64_t stride, const float* gate_bias, float* state, int H, int d,
                      int dv, float cap, const int32_t* cu, const int32_t* slots, const int32_t* pos, int n_seg, int q_off,
                      int k_off, int v_off, int g_off, hipStream_t stream) {
@@ -396,8 +406,8 @@ bool launch_mlstm_vt(float* out, const T* proj, int64_t stride, const float* gat
   const dim3 grid((unsigned)((dv + VT - 1) / VT), (unsigned)H, (unsigned)n_seg);
 #define NGA_MLSTM_CASE(N)                                                                                            \
   if (nr <= N) {                                                                                                     \
-    mlstm_scan_kernel<T, N, VT><<<grid, 256, 0, stream>>>(out, proj, stride, gate_bias, state, H, d, dv, cap, cu, slots, \
-                                                          pos, q_off, k_off, v_off, g_off);                          \
+    mlstm_scan_kernel<T, N, VT, TCN><<<grid, 256, 0, stream>>>(out, proj, stride, gate_bias, state, H, d, dv, cap, cu, \
+                                                               slots, pos, q_off, k_off, v_off, g_off);              \
     return true;                                                                                                     \
   }
   // at most 256 padded rows per head in LDS: NR <= 64 / 32 / 16 for tiles of 64 / 32 / 16 columns
@@ -422,9 +432,14 @@ bool launch_mlstm_t(float* out, const T* proj, int64_t stride, const float* gate
   int vt = dv <= 16 ? 16 : (dv <= 32 ? 32 : 64);
   while (vt > 16 && base * ((dv + vt - 1) / vt) < 1024) vt /= 2;
 #define NGA_MLSTM_ARGS out, proj, stride, gate_bias, state, H, d, dv, cap, cu, slots, pos, n_seg, q_off, k_off, v_off, g_off, stream
-  if (vt == 64 && launch_mlstm_vt<T, 64>(NGA_MLSTM_ARGS)) return true;
-  if (vt >= 32 && launch_mlstm_vt<T, 32>(NGA_MLSTM_ARGS)) return true;
-  return launch_mlstm_vt<T, 16>(NGA_MLSTM_ARGS);
+  if (cu == nullptr) {   // every segment is one row: one row staged per pass
+    if (vt == 64 && launch_mlstm_vt<T, 64, 1>(NGA_MLSTM_ARGS)) return true;
+    if (vt >= 32 && launch_mlstm_vt<T, 32, 1>(NGA_MLSTM_ARGS)) return true;
+    return launch_mlstm_vt<T, 16, 1>(NGA_MLSTM_ARGS);
+  }
+  if (vt == 64 && launch_mlstm_vt<T, 64, TC>(NGA_MLSTM_ARGS)) return true;
+  if (vt >= 32 && launch_mlstm_vt<T, 32, TC>(NGA_MLSTM_ARGS)) return true;
+  return launch_mlstm_vt<T, 16, TC>(NGA_MLSTM_ARGS);
 #undef NGA_MLSTM_ARGS
 }
 

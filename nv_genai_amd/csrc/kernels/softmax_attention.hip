@@ -219,9 +219,11 @@ __global__ void __launch_bounds__(64) softmax_attention_kernel(
 // lanes. The softmax runs per query column in the exp2 domain: the running maximum and sum are
 // reduced over the lane's 16 scores and the 4 lanes of its column; accumulators are rescaled
 // when the maximum moves. Pages visited: those the block's windows cover.
-// tanh on the hardware exp2 and reciprocal (soft cap of the scores in the MFMA kernels)
-__device__ __forceinline__ float tanh_fast(float x) {
-  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(2.8853900817779268f * x));
+// Soft cap of a score in the exp2 domain on the hardware exp2 and reciprocal:
+// cap_log2 * tanh(x) with x = dot * scale / cap, as cap_log2 - 2 cap_log2 / (1 + 2^(k dot)),
+// k = 2 log2(e) * scale / cap (five vector operations per score)
+__device__ __forceinline__ float capped_score(float dot, float k, float cap_log2, float m2cap) {
+  return m2cap * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(k * dot)) + cap_log2;
 }
 
 __device__ __forceinline__ int sm_row_swz(int row) { return (row & 3) | (((row >> 3) & 3) << 2); }
@@ -376,7 +378,7 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
     const float fd = (float)(qpos - kbase - 8 * h);
     const bool need_mask = kbase + KT - 1 > wq_lo || (W > 0 && wq_hi - kbase >= W);
     const bool capped = P.cap_log2 > 0.f;
-    const float inv_cap = capped ? 1.0f / P.cap_log2 : 0.f;
+    const float cap_k = capped ? 2.8853900817779268f * P.scale_log2 / P.cap_log2 : 0.f, cap_m2 = -2.0f * P.cap_log2;
     bf16x8 pf[MAPS][2];
     f32x4 sboth[SHARE ? MAPS : 1][4];
     if constexpr (SHARE) {   // both heads' scores from one read of every K fragment
@@ -420,7 +422,7 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
           float sv = sacc[tau][rr] * P.scale_log2;
-          if (capped) sv = P.cap_log2 * tanh_fast(sv * inv_cap);
+          if (capped) sv = capped_score(sacc[tau][rr], cap_k, P.cap_log2, cap_m2);
           if (need_mask) {
             const float d = fd - (float)(32 * (tau >> 1) + 4 * (tau & 1) + rr);
             sv = (d >= 0.f && d < fW) ? sv : -INFINITY;
@@ -698,7 +700,7 @@ __device__ __forceinline__ void softmax_decode_mfma_body(
     const int kbase = pg * KT;
     const bool need_mask = kbase < lo || kbase + KT - 1 > i;
     const bool capped = cap_log2 > 0.f;
-    const float inv_cap = capped ? 1.0f / cap_log2 : 0.f;
+    const float cap_k = capped ? 2.8853900817779268f * scale_log2 / cap_log2 : 0.f, cap_m2 = -2.0f * cap_log2;
     bf16x8 pf[MAPS][2];
 #pragma unroll
     for (int m = 0; m < MAPS; ++m) {
@@ -723,7 +725,7 @@ __device__ __forceinline__ void softmax_decode_mfma_body(
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
           float sv = sacc[tau][rr] * scale_log2;
-          if (capped) sv = cap_log2 * tanh_fast(sv * inv_cap);
+          if (capped) sv = capped_score(sacc[tau][rr], cap_k, cap_log2, cap_m2);
           if (need_mask) {
             const int j = kbase + 32 * (tau >> 1) + 8 * h + 4 * (tau & 1) + rr;
             sv = (j >= lo && j <= i) ? sv : -INFINITY;
