@@ -210,6 +210,27 @@ bool launch_hgrn2_t(float* out, const T* proj, int64_t stride, const float* f_bi
 // cu == nullptr: segment b is row b. Padded state rows (i >= d) see k = q = 0 and stay 0.
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
+// The gate functions of the scan, all in fp32. PRECISE (fp32 activations): the library functions.
+// Otherwise (bf16 activations) the same formulas on the hardware exp2 / log2 / reciprocal (about
+// 1 ulp each): the gate phase of a pass is a serial stretch in which three of the four waves wait.
+template <bool PRECISE> struct GateMath;
+template <> struct GateMath<true> {
+  static __device__ __forceinline__ float exp(float x) { return expf(x); }
+  static __device__ __forceinline__ float tanh(float x) { return tanhf(x); }
+  static __device__ __forceinline__ float logsig(float z) { return log_sigmoid(z); }
+};
+template <> struct GateMath<false> {
+  static __device__ __forceinline__ float exp(float x) { return __builtin_amdgcn_exp2f(1.4426950408889634f * x); }
+  static __device__ __forceinline__ float tanh(float x) {
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(2.8853900817779268f * x));
+  }
+  // min(z, 0) - ln(1 + e^(-|z|)); the sum 1 + e^(-|z|) lies in (1, 2], so the logarithm loses nothing
+  static __device__ __forceinline__ float logsig(float z) {
+    const float e = __builtin_amdgcn_exp2f(-1.4426950408889634f * fabsf(z));
+    return fminf(z, 0.f) - 0.6931471805599453f * __builtin_amdgcn_logf(1.0f + e);
+  }
+};
+
 // TCN: rows staged per pass (16 for prompt portions; 1 for launches whose segments are single rows: a
 // sixteenth of the LDS, so that all workgroups of a decode step are resident at once)
 template <typename T, int NR, int VT, int TCN>
@@ -220,6 +241,7 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
                                                          const int32_t* __restrict__ slots,
                                                          const int32_t* __restrict__ pos, int q_off, int k_off,
                                                          int v_off, int g_off) {
+  using GM = GateMath<sizeof(T) == 4>;
   constexpr int RG = 256 / VT;
   constexpr int DP = RG * NR;              // padded rows of a head
   constexpr int NQ = (TCN * DP + 255) / 256;   // q (and k) elements a thread stages per pass
@@ -303,8 +325,8 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
       if (e < TCN * VT) vs[e] = rv[x];
     }
     if (tid < TCN) {
-      gi[tid] = cap * tanhf((ri + gate_bias[h]) * inv_cap);
-      gf[tid] = log_sigmoid(cap * tanhf((rf + gate_bias[H + h]) * inv_cap));
+      gi[tid] = cap * GM::tanh((ri + gate_bias[h]) * inv_cap);
+      gf[tid] = GM::logsig(cap * GM::tanh((rf + gate_bias[H + h]) * inv_cap));
     }
     __syncthreads();
     if (tid < 64) {   // the gate chain of the pass on the first wave, one row per lane: the running
@@ -330,9 +352,9 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
       float mp = __shfl_up(m, 1, 64);
       if (tid == 0) mp = m0;
       if (tid < nt) {
-        ga[tid] = expf(f_t + mp - m);
-        gb[tid] = expf(i_t - m);
-        gem[tid] = expf(-m);
+        ga[tid] = GM::exp(f_t + mp - m);
+        gb[tid] = GM::exp(i_t - m);
+        gem[tid] = GM::exp(-m);
       }
       if (tid == TCN - 1) m_carry = m;      // (lanes past nt pass the last row's maximum on)
     }
