@@ -251,7 +251,6 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
   __shared__ float vs[TCN * VT];
   __shared__ float part[TCN * 256];
   __shared__ float partn[TCN * RG];
-  __shared__ float gi[TCN], gf[TCN];         // log gates of the pass
   __shared__ float ga[TCN], gb[TCN], gem[TCN];   // decay of the old state, weight of the new row, e^(-m)
   __shared__ float m_carry;
   const int vt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -324,19 +323,15 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ out
       const int e = tid + 256 * x;
       if (e < TCN * VT) vs[e] = rv[x];
     }
-    if (tid < TCN) {
-      gi[tid] = cap * GM::tanh((ri + gate_bias[h]) * inv_cap);
-      gf[tid] = GM::logsig(cap * GM::tanh((rf + gate_bias[H + h]) * inv_cap));
-    }
-    __syncthreads();
-    if (tid < 64) {   // the gate chain of the pass on the first wave, one row per lane: the running
-      // maximum m_t = max(f_t + m_(t-1), i_t) is a prefix scan over the maps m -> max(m + A, B),
-      // composed as (A1, B1) then (A2, B2) = (A1 + A2, max(B1 + A2, B2)); lanes past the pass's
-      // rows hold the identity. The three exponentials of all rows are then taken side by side.
+    if (tid < 64) {   // the gate chain of the pass on the first wave, one row per lane, straight from the
+      // lane's registers: the running maximum m_t = max(f_t + m_(t-1), i_t) is a prefix scan over the
+      // maps m -> max(m + A, B), composed as (A1, B1) then (A2, B2) = (A1 + A2, max(B1 + A2, B2));
+      // lanes past the pass's rows hold the identity. The three exponentials of all rows are then
+      // taken side by side.
       float A = 0.f, B = -INFINITY;
       if (tid < nt) {
-        A = gf[tid];
-        B = gi[tid];
+        B = cap * GM::tanh((ri + gate_bias[h]) * inv_cap);
+        A = GM::logsig(cap * GM::tanh((rf + gate_bias[H + h]) * inv_cap));
       }
       const float f_t = A, i_t = B;
 #pragma unroll
