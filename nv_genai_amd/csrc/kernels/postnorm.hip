@@ -306,6 +306,46 @@ __global__ void __launch_bounds__(256) group_rmsnorm_kernel(T* __restrict__ out,
   }
 }
 
+// groups of gs % 4 == 0 columns, 16-byte aligned fp32 rows, 8-byte aligned outputs and gates: half a
+// wave per (row, group), four neighbouring elements per lane (16-byte loads of x and w, 8-byte
+// loads of the gate and stores); the sum of squares is reduced inside the half wave
+__global__ void __launch_bounds__(256) group_rmsnorm_bf16x4_kernel(uint16_t* __restrict__ out, const float* __restrict__ x,
+                                                                   const float* __restrict__ w, int64_t n_groups, int gs,
+                                                                   float eps, int groups, int w_full,
+                                                                   const uint16_t* __restrict__ gate, int64_t g_stride) {
+  const int64_t g = blockIdx.x * (int64_t)(blockDim.x >> 5) + (threadIdx.x >> 5);
+  const bool live = g < n_groups;
+  const int sub = threadIdx.x & 31;
+  const int64_t gg = live ? g : 0;
+  const float* xr = x + gg * gs;
+  const int64_t row = gg / groups;
+  const int hg = (int)(gg - row * groups);
+  const float* wr = w_full ? w + (int64_t)hg * gs : w;
+  const uint16_t* gr = gate ? gate + row * g_stride + (int64_t)hg * gs : nullptr;
+  float ss = 0.f;
+  for (int c = 4 * sub; c < gs; c += 128) {
+    const float4 v = *reinterpret_cast<const float4*>(xr + c);
+    ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+  }
+#pragma unroll
+  for (int o = 16; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);   // stays inside the half wave
+  if (!live) return;
+  const float r = 1.0f / sqrtf(ss / (float)gs + eps);
+  for (int c = 4 * sub; c < gs; c += 128) {
+    const float4 v = *reinterpret_cast<const float4*>(xr + c), ww = *reinterpret_cast<const float4*>(wr + c);
+    float y[4] = {v.x * r * ww.x, v.y * r * ww.y, v.z * r * ww.z, v.w * r * ww.w};
+    if (gr) {
+      const u16x4 g4 = *reinterpret_cast<const u16x4*>(gr + c);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) y[q] *= __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * bf2f(g4[q])));
+    }
+    u16x4 o4;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) o4[q] = f2bf(y[q]);
+    *reinterpret_cast<u16x4*>(out + gg * gs + c) = o4;
+  }
+}
+
 // ---- dynamic tanh in place of a norm: tanh(alpha x) * w + b, no statistics
 // rows: gather (nullptr: all rows)
 template <typename T>
@@ -574,6 +614,12 @@ void launch_group_rmsnorm(void* out, const float* x, const float* w, bool w_full
                           int64_t T, int groups, int gs, float eps, bool f32, hipStream_t stream) {
   const int64_t ng = T * groups;
   if (ng == 0) return;
+  if (!f32 && gs % 4 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)out % 8) == 0 &&
+      (gate == nullptr || (g_stride % 4 == 0 && ((uintptr_t)gate % 8) == 0))) {
+    group_rmsnorm_bf16x4_kernel<<<dim3((unsigned)((ng + 7) / 8)), 256, 0, stream>>>(
+        (uint16_t*)out, x, w, ng, gs, eps, groups, w_full ? 1 : 0, (const uint16_t*)gate, g_stride);
+    return;
+  }
   const unsigned g = (unsigned)((ng + 3) / 4);
   const int pair = (gs % 2 == 0 && ((uintptr_t)x % 8) == 0) ? 1 : 0;
   if (f32)
